@@ -1,0 +1,170 @@
+/*
+ * triton_int_hip.h — C ABI of libtriton_int_hip.so (gfx950 / MI355X only).
+ *
+ * Every entry point takes raw device pointers, element strides, sizes and a HIP
+ * stream handle (passed as void*; NULL = the null stream).  Nothing here knows
+ * about torch.  All calls only enqueue work on `stream` and return; there is no
+ * host synchronisation.  Return value: 0 = ok, <0 = invalid argument (TI_E_*),
+ * >0 = a hipError_t from the launch.  ti_last_error() returns a thread-local
+ * message for the last non-zero return.
+ *
+ * Each entry point names the reference interface (file:line in
+ * zhanglei1172/triton_int) whose Triton launch it replaces.
+ *
+ * Arithmetic contract shared by all GEMM/BMM epilogues:
+ *   acc      exact int32  sum_k a[m,k] * b[n,k]
+ *   f(.)     int32 -> fp32 conversion, round-to-nearest-even
+ *   all fp32 products and sums are separately rounded (no FMA contraction)
+ *   q8(v)    TI_ROUND_RNE_CLAMP: clamp(round_half_even(v), -128, 127), NaN -> 0
+ *            TI_ROUND_TRUNC    : clamp(trunc(v), -128, 127)  (literal Triton `.to(int8)`
+ *                                on in-range values; test-time switch only)
+ */
+#ifndef TRITON_INT_HIP_H
+#define TRITON_INT_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- enums (plain ints in the ABI) ------------------------------------------------- */
+
+enum ti_epilogue {
+  /* C_i32 = acc (+ bias_i32[n])
+   *   kernels/linear.py:433-566 (linear_a8_w8_b32_o32), kernels/bmm.py:163-311
+   *   (bmm_s8t_s8n_s32t), kernels/bmm.py:12-160 (bmm_s8t_s8t_s32t) */
+  TI_EPI_I32 = 0,
+  /* C_i32 = cvt_i32(alpha*f(acc) + beta*f(bias_i32[n]))
+   *   kernels/linear.py:569-708 (linear_a8_w8_b32_o32_with_scaling) */
+  TI_EPI_SCALE_I32 = 1,
+  /* C_i8 = q8(alpha*f(acc) + beta*f(bias_i8[n]))   (bias optional)
+   *   kernels/linear.py:150-288 (linear_a8_w8_b8_o8), kernels/bmm.py:467-612
+   *   (bmm_s8t_s8n_s8t), kernels/bmm.py:615-760 (bmm_s8t_s8t_s8t) */
+  TI_EPI_SCALE_I8 = 2,
+  /* C_i8 = max(q8(...), 0)   kernels/linear.py:291-430 (linear_relu_a8_w8_b8_o8) */
+  TI_EPI_SCALE_RELU_I8 = 3,
+  /* C_f = alpha*f(acc) + beta*bias_f32[n]  -> f32 / f16 / bf16   (bias optional)
+   *   kernels/linear.py:711-853 (linear_a8_w8_bfp32_ofp32), kernels/linear.py:24-147
+   *   (linear_a8_w8_ofp32), kernels/bmm.py:314-464 (bmm_s8t_s8n_f32t) */
+  TI_EPI_SCALE_F = 4,
+  /* x = alpha*f(acc) + bias_f32[n];  C_i8 = q8(0.5*x*(1+tanh(sqrt(2/pi)*(x+0.044715*x^3)))*beta)
+   *   kernels/fused.py:76-79,88-231 (linear_a8_w8_bfp32_ofp32_GeLu_Q) */
+  TI_EPI_GELU_I8 = 5,
+  TI_EPI_COUNT_ = 6
+};
+
+enum ti_dtype { TI_I8 = 0, TI_I32 = 1, TI_F32 = 2, TI_F16 = 3, TI_BF16 = 4 };
+enum ti_bias { TI_BIAS_NONE = 0, TI_BIAS_I8 = 1, TI_BIAS_I32 = 2, TI_BIAS_F32 = 3 };
+enum ti_round { TI_ROUND_RNE_CLAMP = 0, TI_ROUND_TRUNC = 1 };
+
+enum ti_status {
+  TI_OK = 0,
+  TI_E_NULL = -1,      /* a required pointer is NULL */
+  TI_E_SHAPE = -2,     /* negative size, or size beyond what the kernels index with int32 */
+  TI_E_COMBO = -3,     /* epilogue / out dtype / bias kind combination not defined */
+  TI_E_STRIDE = -4,    /* stride not usable (zero/negative stride on an output, ...) */
+  TI_E_DEVICE = -5     /* current device is not gfx950 */
+};
+
+/* ---- library ----------------------------------------------------------------------- */
+
+/* ABI version, bumped when a signature changes. */
+int ti_version(void);
+/* Message for the last non-zero status returned on the calling thread ("" if none). */
+const char* ti_last_error(void);
+
+/* ---- int8 GEMM / BMM --------------------------------------------------------------- */
+
+/*
+ * Batched C[b,m,n] = epilogue( sum_k A[b,m,k] * B[b,n,k] ).
+ *
+ * Replaces every int8 Triton launcher in kernels/linear.py:117-853, kernels/bmm.py:125-760
+ * and kernels/fused.py:197-231.  A linear is batch = 1.  All strides are in ELEMENTS and
+ * arbitrary (the reference forwards tensor strides, kernels/linear.py:281-286,
+ * kernels/bmm.py:139-151); the "[B,K,N]" operand of bmm_s8t_s8t_* is expressed by
+ * sBn = 1, sBk = N.  The fastest kernels are used when sAk == sBk == 1, K % 16 == 0,
+ * row/batch strides are multiples of 16 and base pointers are 16-byte aligned; any other
+ * stride pattern runs a slower byte-gather kernel with identical results.
+ *
+ * alpha, beta: DEVICE pointers to one fp32 each (the reference loads its 0-dim scale
+ * tensors inside the kernel, kernels/linear.py:227,247).  beta may be NULL when bias is
+ * TI_BIAS_NONE; alpha may be NULL for TI_EPI_I32.
+ * bias: device pointer to N contiguous elements of `bias_kind`, or NULL/TI_BIAS_NONE.
+ * M, N or batch equal to 0 is a no-op; K == 0 gives acc = 0.
+ */
+int ti_bmm_i8(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk,
+              const int8_t* B, int64_t sBb, int64_t sBn, int64_t sBk,
+              void* C, int64_t sCb, int64_t sCm, int64_t sCn,
+              int batch, int M, int N, int K,
+              const void* bias, int bias_kind,
+              const float* alpha, const float* beta,
+              int epilogue, int out_dtype, int round_mode,
+              void* stream);
+
+/*
+ * Same as ti_bmm_i8 but forces one kernel configuration (index into the library's tile
+ * table; see ti_gemm_num_configs / ti_gemm_config_name).  Used by the tuner and the
+ * parity tests so that every configuration is checked, not only the one the dispatcher
+ * would pick.  config = -1 selects automatically.  Returns TI_E_COMBO if the
+ * configuration cannot run the given stride pattern.
+ */
+int ti_bmm_i8_config(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk,
+                     const int8_t* B, int64_t sBb, int64_t sBn, int64_t sBk,
+                     void* C, int64_t sCb, int64_t sCm, int64_t sCn,
+                     int batch, int M, int N, int K,
+                     const void* bias, int bias_kind,
+                     const float* alpha, const float* beta,
+                     int epilogue, int out_dtype, int round_mode,
+                     int config, void* stream);
+int ti_gemm_num_configs(void);
+const char* ti_gemm_config_name(int config);
+
+/* ---- row kernels ------------------------------------------------------------------- */
+
+/*
+ * y_i8[r,:] = q8( ((x[r,:] - mean_r) * rstd_r) * gamma + beta ),  rstd = 1/sqrt(var + eps),
+ * biased variance; rms != 0 selects the RMSNorm branch (mean = 0, var = mean(x^2)).
+ * Replaces layer_norm_fwd_fused_single_pass_q, kernels/fused.py:235-382 (module LayerNormQ,
+ * nn/fused.py:34-57).  x is fp32 with unit column stride and row stride `x_row_stride`
+ * elements; y has row stride `y_row_stride`.  beta may be NULL (HAS_BIAS = False,
+ * kernels/fused.py:324-326).  mean_out / rstd_out (fp32[rows], may be NULL) receive the row
+ * statistics for tests.
+ */
+int ti_layernorm_q(const float* x, int64_t x_row_stride,
+                   const float* gamma, const float* beta, float eps,
+                   int8_t* y, int64_t y_row_stride,
+                   int rows, int cols, int rms, int round_mode,
+                   float* mean_out, float* rstd_out, void* stream);
+
+/*
+ * resid_out = resid_in + in_scale * f(acc_i32);  y_i8 = q8(LayerNorm(resid_out; gamma, beta, eps)).
+ * The native op the reference intends at functional/fused.py:27-32 (module
+ * DQ_Add_LayerNorm_Q, nn/fused.py:59-78) and defines only as the PyTorch emulation
+ * functional/fused.py:6-15.  in_scale is a host float (nn/fused.py:62,73).  All row-major
+ * with unit column stride; row strides in elements.  resid_out may alias resid_in.
+ * ln_out_f32 (may be NULL) additionally receives the fp32 LayerNorm output, which is what
+ * the un-quantised variant returns (functional/fused.py:18-24, dq_add_layernorm); y may be
+ * NULL when only that variant is wanted.  At least one of y / ln_out_f32 must be given.
+ */
+int ti_dq_add_layernorm_q(const int32_t* acc, int64_t acc_row_stride, float in_scale,
+                          const float* resid_in, int64_t resid_in_row_stride,
+                          const float* gamma, const float* beta, float eps,
+                          float* resid_out, int64_t resid_out_row_stride,
+                          int8_t* y, int64_t y_row_stride,
+                          float* ln_out_f32, int64_t ln_out_row_stride,
+                          int rows, int cols, int round_mode,
+                          float* mean_out, float* rstd_out, void* stream);
+
+/*
+ * y_i8[i] = q8( 0.5*x*(1+tanh(sqrt(2/pi)*(x+0.044715*x^3))) * scale ),  i < n, contiguous.
+ * Stand-alone form of fast_geluQ, kernels/fused.py:76-79 (module GeLu_Q, nn/fused.py:81-87).
+ * scale: DEVICE pointer to one fp32.
+ */
+int ti_gelu_q(const float* x, const float* scale, int8_t* y, int64_t n,
+              int round_mode, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TRITON_INT_HIP_H */

@@ -1,0 +1,140 @@
+"""Pins for the oracle's LayerNormQ, dq+add+LayerNormQ and GELU-quant restatements against
+torch's own library routines (the calls the reference's CPU emulation makes:
+functional/fused.py:6-15, nn/fused.py:15-22) and against closed forms."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle as O
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+def torch_lnq(x, w, b, eps):
+    y = F.layer_norm(torch.from_numpy(x), (x.shape[-1],), torch.from_numpy(w), None if b is None else torch.from_numpy(b), eps)
+    return y.round().clamp(-128, 127).to(torch.int8).numpy(), y.numpy()
+
+
+@pytest.mark.parametrize("cols", [1, 7, 128, 768, 5120])
+def test_layernorm_q_vs_torch_layer_norm(cols):
+    g = rng(cols)
+    rows = 33
+    x = (g.standard_normal((rows, cols)) * 1.7 + 0.3).astype(np.float32)
+    w = (g.normal(1.0, 0.1, cols) / 0.05).astype(np.float32)
+    b = (g.normal(0.0, 0.1, cols) / 0.05).astype(np.float32)
+    got, mean, rstd = O.layernorm_q(x, w, b, 1e-5, return_stats=True)
+    want, yf = torch_lnq(x, w, b, 1e-5)
+    # statistics against float64
+    x64 = x.astype(np.float64)
+    assert np.allclose(mean, x64.mean(1), rtol=0, atol=1e-6)
+    assert np.allclose(rstd, 1.0 / np.sqrt(x64.var(1) + 1e-5), rtol=2e-6)
+    diff = np.abs(got.astype(np.int32) - want.astype(np.int32))
+    assert diff.max() <= 1
+    # only values sitting on a rounding boundary may differ (summation-order ulps)
+    frac = np.abs(yf - np.floor(yf) - 0.5)
+    assert np.all(frac[diff != 0] < 2e-3)
+    assert (diff != 0).mean() < 1e-3
+    # fp64 layer_norm as the tie-breaker: the oracle must agree with it wherever not near a tie
+    y64 = F.layer_norm(torch.from_numpy(x64), (cols,), torch.from_numpy(w).double(), torch.from_numpy(b).double(), 1e-5)
+    want64 = y64.round().clamp(-128, 127).to(torch.int8).numpy()
+    safe = np.abs(y64.numpy() - np.floor(y64.numpy()) - 0.5) > 1e-3
+    assert np.array_equal(got[safe], want64[safe])
+
+
+def test_layernorm_q_no_bias_and_rms():
+    g = rng(11)
+    x = g.standard_normal((9, 320)).astype(np.float32) * 3
+    w = (g.normal(1.0, 0.1, 320) * 20).astype(np.float32)
+    got = O.layernorm_q(x, w, None, 1e-5)
+    want, _ = torch_lnq(x, w, None, 1e-5)
+    assert np.abs(got.astype(int) - want.astype(int)).max() <= 1 and (got != want).mean() < 1e-3
+    # RMSNorm branch (kernels/fused.py:291-292,307-308): mean stays 0, var = mean(x^2)
+    got_r, mean, rstd = O.layernorm_q(x, w, None, 1e-5, rms=True, return_stats=True)
+    x64 = x.astype(np.float64)
+    r64 = 1.0 / np.sqrt((x64 ** 2).mean(1) + 1e-5)
+    assert np.all(mean == 0) and np.allclose(rstd, r64, rtol=2e-6)
+    y64 = x64 * r64[:, None] * w.astype(np.float64)
+    safe = np.abs(y64 - np.floor(y64) - 0.5) > 1e-3
+    assert np.array_equal(got_r[safe], np.clip(np.rint(y64), -128, 127).astype(np.int8)[safe])
+
+
+def test_layernorm_constant_row_and_large_offset():
+    cols = 256
+    w = np.full(cols, 10.0, np.float32)
+    b = np.full(cols, 3.0, np.float32)
+    x = np.full((2, cols), 5.0, np.float32)
+    got, mean, rstd = O.layernorm_q(x, w, b, 1e-5, return_stats=True)
+    assert np.all(mean == 5.0) and np.allclose(rstd, 1 / np.sqrt(1e-5), rtol=1e-6)
+    assert np.all(got == 3)  # (x-mean) == 0 exactly -> bias only
+    # shift invariance: adding a large representable offset leaves the result unchanged
+    g = rng(12)
+    base = g.integers(-64, 64, size=(4, cols)).astype(np.float32) / 8  # exact in fp32 after +1e4
+    q0 = O.layernorm_q(base, w, b, 1e-5)
+    q1 = O.layernorm_q(base + np.float32(1e4), w, b, 1e-5)
+    assert np.array_equal(q0, q1)
+
+
+def test_dq_add_layernorm_q_vs_torch_emulation_calls():
+    g = rng(13)
+    rows, cols = 17, 5120
+    acc = g.integers(-2**20, 2**20 + 1, size=(rows, cols), dtype=np.int32)
+    acc[0, :4] = [2**20, -2**20, 0, 1]
+    s = 1e-5
+    res = g.standard_normal((rows, cols)).astype(np.float32)
+    w = (g.normal(1.0, 0.1, cols) / 0.05).astype(np.float32)
+    b = (g.normal(0.0, 0.1, cols) / 0.05).astype(np.float32)
+    rout, q, ln, mean, rstd = O.dq_add_layernorm_q(acc, s, res, w, b, 1e-5, return_all=True)
+    # the emulation's own calls
+    t_res = torch.add(torch.from_numpy(res), torch.from_numpy(acc), alpha=s)
+    t_ln = F.layer_norm(t_res, (cols,), torch.from_numpy(w), torch.from_numpy(b), 1e-5)
+    t_q = t_ln.clamp(-128, 127).round().to(torch.int8).numpy()
+    assert np.allclose(rout, t_res.numpy(), rtol=1e-6, atol=1e-7)      # FMA vs mul+add: <= 1 ulp
+    assert np.allclose(ln, t_ln.numpy(), rtol=1e-5, atol=2e-5)
+    diff = np.abs(q.astype(int) - t_q.astype(int))
+    assert diff.max() <= 1 and (diff != 0).mean() < 1e-3
+    # exactness of the un-fused dequant: resid_out == fl(res + fl(s*x))
+    p = (np.float32(s) * acc.astype(np.float32)).astype(np.float32)
+    assert np.array_equal(rout, res + p)
+    x64 = rout.astype(np.float64)
+    assert np.allclose(mean, x64.mean(1), atol=1e-6)
+    assert np.allclose(rstd, 1 / np.sqrt(x64.var(1) + 1e-5), rtol=2e-6)
+
+
+def test_dq_add_exact_when_representable():
+    # s = 2^-10 and small ints: s*x and the sum are exact, so resid_out - resid_in == s*x exactly
+    acc = np.arange(-512, 512, dtype=np.int32).reshape(4, 256)
+    res = np.full((4, 256), 0.25, np.float32)
+    w = np.ones(256, np.float32); b = np.zeros(256, np.float32)
+    rout, _ = O.dq_add_layernorm_q(acc, 2.0 ** -10, res, w, b, 1e-5)
+    assert np.array_equal(rout - res, acc.astype(np.float32) * np.float32(2.0 ** -10))
+
+
+def test_gelu_q_vs_torch_and_closed_forms():
+    x = np.linspace(-8, 8, 20001).astype(np.float32)
+    scale = np.float32(1 / 0.05)
+    got = O.gelu_q(x, scale)
+    yf = (F.gelu(torch.from_numpy(x), approximate="tanh") * torch.tensor(scale))
+    want = yf.round().clamp(-128, 127).to(torch.int8).numpy()
+    diff = np.abs(got.astype(int) - want.astype(int))
+    assert diff.max() <= 1
+    frac = np.abs(yf.numpy() - np.floor(yf.numpy()) - 0.5)
+    assert np.all(frac[diff != 0] < 1e-3)
+    # closed forms on the un-quantised value
+    one = np.float32(1.0)
+    assert O.gelu_f32(np.zeros(1, np.float32), one)[0] == 0.0
+    big = np.array([9.0, 20.0, 100.0], np.float32)
+    assert np.array_equal(O.gelu_f32(big, one), big)             # tanh saturates to 1: gelu(x) = x
+    assert np.all(np.abs(O.gelu_f32(-big, one)) == 0.0)          # and to -1: gelu(-x) = 0
+    xs = np.linspace(0.01, 6, 997).astype(np.float32)
+    odd = O.gelu_f32(xs, one).astype(np.float64) - O.gelu_f32(-xs, one).astype(np.float64)
+    assert np.allclose(odd, xs, rtol=0, atol=1e-6)               # gelu(x) - gelu(-x) = x
+    # float64 evaluation of the same closed form
+    x64 = xs.astype(np.float64)
+    ref = 0.5 * x64 * (1 + np.tanh(np.sqrt(2 / np.pi) * (x64 + 0.044715 * x64 ** 3)))
+    assert np.allclose(O.gelu_f32(xs, one), ref, rtol=2e-6, atol=1e-7)
+    # saturation of the quantiser
+    assert O.gelu_q(np.array([100.0], np.float32), scale)[0] == 127
+    assert O.gelu_q(np.array([-0.75], np.float32), np.float32(1000.0))[0] == -128
