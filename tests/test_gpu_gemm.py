@@ -1,0 +1,277 @@
+"""GPU parity of the int8 GEMM / BMM kernels against the CPU oracle, called through the package's
+launchers (which go through the C ABI).  int32 and scale epilogues must be bit-exact; the GELU
+epilogue may differ by 1 LSB where tanh's last ulp decides a rounding tie (rate asserted)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from tests.util import DEV, cpu, gpu, mismatch_report, rand_i8, rng
+
+pytestmark = pytest.mark.gpu
+
+
+def _lib():
+    from triton_int_amd import _lib as L
+    return L
+
+
+def _configs():
+    L = _lib()
+    n = L.lib().ti_gemm_num_configs()
+    return [(i, L.lib().ti_gemm_config_name(i).decode()) for i in range(n)]
+
+
+def _kl():
+    from triton_int_amd.kernels import linear, bmm, fused
+    return linear, bmm, fused
+
+
+# shapes: (M, N, K); all K % 16 == 0 so that every configuration can run them
+SHAPES = [(512, 768, 768), (300, 272, 384), (256, 128, 128), (33, 100, 48), (1, 16, 16), (700, 130, 1040)]
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_all_configs_int32_bit_exact(shape):
+    linear, _, _ = _kl()
+    M, N, K = shape
+    g = rng(M * 7 + N)
+    a, w = rand_i8(g, M, K, lo=-128), rand_i8(g, N, K, lo=-128)
+    bias = g.integers(-2**24, 2**24, size=N, dtype=np.int32)
+    want = O.linear_a8_w8_b32_o32(a, w, bias)
+    ga, gw, gb = gpu(a), gpu(w), gpu(bias)
+    for cfg, name in _configs():
+        got = cpu(linear.linear_a8_w8_b32_o32(ga, gw, gb, _config=cfg))
+        assert np.array_equal(got, want), f"config {name}"
+    got = cpu(linear.linear_a8_w8_b32_o32(ga, gw, gb))
+    assert np.array_equal(got, want), "auto config"
+
+
+@pytest.mark.parametrize("shape", SHAPES[:4], ids=lambda s: "x".join(map(str, s)))
+def test_all_configs_int8_epilogues_bit_exact(shape):
+    linear, _, _ = _kl()
+    M, N, K = shape
+    g = rng(M * 3 + K)
+    a, w, bias = rand_i8(g, M, K), rand_i8(g, N, K), rand_i8(g, N)
+    ga, gw, gb = gpu(a), gpu(w), gpu(bias)
+    std = np.sqrt(K) * 127 * 127 / 3
+    for alpha, beta in [(0.0021, 0.013), (40.0 / std, 0.11), (0.5, 1.0)]:  # saturating, spread, exact ties
+        want = O.linear_a8_w8_b8_o8(a, w, bias, alpha, beta)
+        want_relu = O.linear_relu_a8_w8_b8_o8(a, w, bias, alpha, beta)
+        want_tr = O.linear_a8_w8_b8_o8(a, w, bias, alpha, beta, round_mode=O.TRUNC)
+        for cfg, name in _configs():
+            got = cpu(linear.linear_a8_w8_b8_o8(ga, gw, gb, alpha, beta, _config=cfg))
+            assert np.array_equal(got, want), f"o8 config {name} alpha {alpha}"
+            got = cpu(linear.linear_relu_a8_w8_b8_o8(ga, gw, gb, alpha, beta, _config=cfg))
+            assert np.array_equal(got, want_relu), f"relu config {name}"
+        got = cpu(linear.linear_a8_w8_b8_o8(ga, gw, gb, alpha, beta, _round_mode=1))
+        assert np.array_equal(got, want_tr)
+        # the literal-Triton truncation differs from the contract by at most 1 on unsaturated values
+        assert np.abs(want_tr.astype(int) - want.astype(int)).max() <= 1
+
+
+@pytest.mark.parametrize("shape", SHAPES[:4], ids=lambda s: "x".join(map(str, s)))
+def test_all_configs_float_and_scaled_i32(shape):
+    linear, _, _ = _kl()
+    M, N, K = shape
+    g = rng(M + N + K)
+    a, w = rand_i8(g, M, K), rand_i8(g, N, K)
+    bias_f = g.standard_normal(N).astype(np.float32)
+    bias_i = g.integers(-10**6, 10**6, size=N, dtype=np.int32)
+    alpha, beta = np.float32(0.0037), np.float32(0.71)
+    ga, gw = gpu(a), gpu(w)
+    want_f = O.linear_a8_w8_bfp32_ofp32(a, w, bias_f, alpha, beta)
+    want_h = O.linear_a8_w8_bfp32_ofp32(a, w, bias_f, alpha, beta, out_dtype=O.DT_F16)
+    want_b = O.linear_a8_w8_bfp32_ofp32(a, w, bias_f, alpha, beta, out_dtype=O.DT_BF16)
+    want_nb = O.linear_a8_w8_ofp32(a, w, alpha)
+    want_s = O.linear_a8_w8_b32_o32_with_scaling(a, w, bias_i, alpha, beta)
+    for cfg, name in _configs():
+        got = cpu(linear.linear_a8_w8_bfp32_ofp32(ga, gw, gpu(bias_f), alpha, beta, _config=cfg))
+        assert got.dtype == np.float32 and np.array_equal(got, want_f), f"f32 {name}"
+        got = cpu(linear.linear_a8_w8_bfp32_ofp32(ga, gw, gpu(bias_f), alpha, beta, dtype=torch.float16, _config=cfg))
+        assert np.array_equal(got, want_h), f"f16 {name}"
+        got = cpu(linear.linear_a8_w8_bfp32_ofp32(ga, gw, gpu(bias_f), alpha, beta, dtype=torch.bfloat16, _config=cfg))
+        assert np.array_equal(got, want_b), f"bf16 {name}"
+        got = cpu(linear.linear_a8_w8_ofp32(ga, gw, alpha, _config=cfg))
+        assert np.array_equal(got, want_nb), f"ofp32 {name}"
+        got = cpu(linear.linear_a8_w8_b32_o32_with_scaling(ga, gw, gpu(bias_i), alpha, beta, _config=cfg))
+        assert np.array_equal(got, want_s), f"scaled i32 {name}"
+
+
+@pytest.mark.parametrize("shape", SHAPES[:3], ids=lambda s: "x".join(map(str, s)))
+def test_all_configs_gelu_q(shape):
+    _, _, fused = _kl()
+    M, N, K = shape
+    g = rng(K)
+    a, w = rand_i8(g, M, K), rand_i8(g, N, K)
+    bias = g.standard_normal(N).astype(np.float32)
+    alpha = np.float32(3.0 / (np.sqrt(K) * 127 * 127 / 3))
+    beta = np.float32(1 / 0.05)
+    want = O.linear_a8_w8_bfp32_ofp32_GeLu_Q(a, w, bias, alpha, beta)
+    assert np.unique(want).size > 100  # the case really exercises the rounding, not only the clamp
+    ga, gw, gb = gpu(a), gpu(w), gpu(bias)
+    for cfg, name in _configs():
+        got = cpu(fused.linear_a8_w8_bfp32_ofp32_GeLu_Q(ga, gw, gb, alpha, beta, _config=cfg))
+        mx, rate = mismatch_report(got, want)
+        assert mx <= 1 and rate < 1e-3, f"{name}: max {mx} rate {rate}"
+
+
+def test_extreme_accumulators_over_2p24():
+    linear, _, _ = _kl()
+    K = 2048
+    a = np.full((40, K), 127, np.int8)
+    w = np.full((48, K), 127, np.int8)
+    w[1::2] = -128
+    want = O.linear_a8_w8_b32_o32(a, w, None)
+    assert want.max() == K * 127 * 127
+    got = cpu(linear.linear_a8_w8_b32_o32(gpu(a), gpu(w), None))
+    assert np.array_equal(got, want)
+    # int32 -> fp32 conversion must round to nearest even, like the oracle's
+    wantf = O.linear_a8_w8_ofp32(a, w, np.float32(1.0))
+    gotf = cpu(linear.linear_a8_w8_ofp32(gpu(a), gpu(w), 1.0))
+    assert np.array_equal(gotf, wantf)
+
+
+def test_bmm_layouts_strides_and_batch():
+    _, bmm, _ = _kl()
+    g = rng(5)
+    B, M, N, K = 3, 40, 24, 72
+    a_big = rand_i8(g, B, M, K + 8)
+    b = rand_i8(g, B, N, K)
+    a_np = a_big[:, :, 4:4 + K]
+    ga = gpu(a_big)[:, :, 4:4 + K]          # non-contiguous, unaligned rows -> gather kernel
+    gb = gpu(b)
+    gb_kn = gpu(np.ascontiguousarray(b.transpose(0, 2, 1)))
+    want32 = O.bmm_s8t_s8n_s32t(a_np, b)
+    assert np.array_equal(cpu(bmm.bmm_s8t_s8n_s32t(ga, gb)), want32)
+    assert np.array_equal(cpu(bmm.bmm_s8t_s8t_s32t(ga, gb_kn)), want32)
+    alpha = np.float32(1e-3)
+    want8 = O.bmm_s8t_s8n_s8t(a_np, b, alpha)
+    assert np.array_equal(cpu(bmm.bmm_s8t_s8n_s8t(ga, gb, float(alpha))), want8)
+    assert np.array_equal(cpu(bmm.bmm_s8t_s8t_s8t(ga, gb_kn, gpu(np.array(alpha)))), want8)
+    wantf = O.bmm_s8t_s8n_f32t(a_np, b, alpha)
+    assert np.array_equal(cpu(bmm.bmm_s8t_s8n_f32t(ga, gb, alpha)), wantf)
+    got16 = bmm.bmm_s8t_s8n_f32t(ga, gb, alpha, dtype=torch.float16)
+    assert got16.dtype == torch.float16
+    assert np.array_equal(cpu(got16), O.bmm_s8t_s8n_f32t(a_np, b, alpha, out_dtype=O.DT_F16))
+
+
+@pytest.mark.parametrize("B,M,N,K", [(5, 256, 384, 128), (2, 300, 200, 64), (7, 64, 64, 256)])
+def test_bmm_fast_path_all_configs(B, M, N, K):
+    _, bmm, _ = _kl()
+    g = rng(B * M)
+    a, b = rand_i8(g, B, M, K), rand_i8(g, B, N, K)
+    ga, gb = gpu(a), gpu(b)
+    want32 = O.bmm_s8t_s8n_s32t(a, b)
+    alpha = np.float32(1e-3)
+    want8 = O.bmm_s8t_s8n_s8t(a, b, alpha)
+    wantf = O.bmm_s8t_s8n_f32t(a, b, alpha)
+    for cfg, name in _configs():
+        assert np.array_equal(cpu(bmm.bmm_s8t_s8n_s32t(ga, gb, _config=cfg)), want32), name
+        assert np.array_equal(cpu(bmm.bmm_s8t_s8n_s8t(ga, gb, alpha, _config=cfg)), want8), name
+        assert np.array_equal(cpu(bmm.bmm_s8t_s8n_f32t(ga, gb, alpha, _config=cfg)), wantf), name
+
+
+def test_odd_k_and_unaligned_fall_back_to_gather():
+    linear, _, _ = _kl()
+    g = rng(77)
+    for (M, N, K) in [(37, 29, 50), (64, 64, 1), (5, 3, 129)]:
+        a, w = rand_i8(g, M, K), rand_i8(g, N, K)
+        want = O.linear_a8_w8_b32_o32(a, w, None)
+        got = cpu(linear.linear_a8_w8_b32_o32(gpu(a), gpu(w), None))
+        assert np.array_equal(got, want), (M, N, K)
+    # a fast configuration must refuse what it cannot run, not compute garbage
+    a, w = rand_i8(g, 8, 50), rand_i8(g, 8, 50)
+    with pytest.raises(AssertionError):
+        linear.linear_a8_w8_b32_o32(gpu(a), gpu(w), None, _config=1)
+
+
+def test_k_zero_empty_and_errors():
+    linear, bmm, _ = _kl()
+    a = torch.zeros((4, 0), dtype=torch.int8, device=DEV)
+    w = torch.zeros((6, 0), dtype=torch.int8, device=DEV)
+    bias = torch.arange(6, dtype=torch.int32, device=DEV)
+    got = cpu(linear.linear_a8_w8_b32_o32(a, w, bias))
+    assert np.array_equal(got, np.tile(np.arange(6, dtype=np.int32), (4, 1)))
+    assert linear.linear_a8_w8_b32_o32(torch.zeros((0, 16), dtype=torch.int8, device=DEV),
+                                       torch.zeros((6, 16), dtype=torch.int8, device=DEV), None).shape == (0, 6)
+    with pytest.raises(AssertionError, match="Incompatible dimensions"):
+        linear.linear_a8_w8_b32_o32(torch.zeros((4, 16), dtype=torch.int8, device=DEV),
+                                    torch.zeros((4, 32), dtype=torch.int8, device=DEV), None)
+    with pytest.raises(AssertionError):
+        bmm.bmm_s8t_s8n_s32t(torch.zeros((2, 4, 16), dtype=torch.int8, device=DEV),
+                             torch.zeros((3, 4, 16), dtype=torch.int8, device=DEV))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        linear.linear_a8_w8_b32_o32(torch.zeros((4, 16), dtype=torch.int8), torch.zeros((4, 16), dtype=torch.int8), None)
+
+
+def test_out_argument_and_leading_dims():
+    linear, _, _ = _kl()
+    g = rng(9)
+    a, w, bias = rand_i8(g, 2, 3, 5, 64), rand_i8(g, 48, 64), rand_i8(g, 48)
+    want = O.linear_a8_w8_b8_o8(a, w, bias, 0.002, 0.1)
+    out = torch.empty((30, 48), dtype=torch.int8, device=DEV)
+    got = linear.linear_a8_w8_b8_o8(gpu(a), gpu(w), gpu(bias), 0.002, 0.1, out=out)
+    assert got.shape == (2, 3, 5, 48)
+    assert got.data_ptr() == out.data_ptr()
+    assert np.array_equal(cpu(got), want)
+
+
+def test_baseline_config1_single_w8a8b8o8_linear():
+    """x int8 [512,768], W int8 [768,768], bias int8 [768], alpha=0.0021, beta=0.013."""
+    from triton_int_amd.nn.linear import W8A8B8O8Linear
+    g = rng(2024)
+    x, w, bias = rand_i8(g, 512, 768), rand_i8(g, 768, 768), rand_i8(g, 768)
+    m = W8A8B8O8Linear(768, 768, alpha=0.0021, beta=0.013)
+    m.weight, m.bias = torch.from_numpy(w), torch.from_numpy(bias)
+    m = m.to(DEV)
+    got = cpu(m(gpu(x)))
+    want = O.linear_a8_w8_b8_o8(x, w, bias, 0.0021, 0.013)
+    assert np.array_equal(got, want)
+    # the CPU emulation path the baseline names: int32 matmul + the same scaling
+    acc = torch.matmul(torch.from_numpy(x).to(torch.int32), torch.from_numpy(w).to(torch.int32).T)
+    emu = torch.clamp(torch.round(torch.tensor(0.0021) * acc.float() + torch.tensor(0.013) * torch.from_numpy(bias).float()), -128, 127)
+    assert np.array_equal(got, emu.to(torch.int8).numpy())
+    # how much of this mandated case is decided by the clamp alone
+    sat = float(((want == 127) | (want == -128)).mean())
+    assert 0.3 < sat < 0.9
+
+
+@pytest.mark.parametrize("which", ["qkv", "fc1_gelu", "fc2"])
+def test_baseline_config2_opt67b_shapes_sampled_rows(which):
+    """Full OPT-6.7B shapes at M=2048 on the GPU; the oracle checks 24 sampled rows (rows are
+    independent) plus int32 linearity over the whole output."""
+    linear, _, fused = _kl()
+    g = rng({"qkv": 1, "fc1_gelu": 2, "fc2": 3}[which])
+    M = 2048
+    K, N = {"qkv": (4096, 4096), "fc1_gelu": (4096, 16384), "fc2": (16384, 4096)}[which]
+    x, w = rand_i8(g, M, K), rand_i8(g, N, K)
+    alpha = np.float32(g.uniform(1e-3, 1e-2)); beta = np.float32(g.uniform(1e-3, 1e-2))
+    rows = np.sort(g.choice(M, size=24, replace=False))
+    gx, gw = gpu(x), gpu(w)
+    if which == "qkv":
+        bias = rand_i8(g, N)
+        got = cpu(linear.linear_a8_w8_b8_o8(gx, gw, gpu(bias), alpha, beta))
+        assert np.array_equal(got[rows], O.linear_a8_w8_b8_o8(x[rows], w, bias, alpha, beta))
+        # non-saturating scale so that rounding is exercised, not only the clamp
+        a2 = np.float32(40.0 / (np.sqrt(K) * 127 * 127 / 3))
+        got2 = cpu(linear.linear_a8_w8_b8_o8(gx, gw, gpu(bias), a2, beta))
+        want2 = O.linear_a8_w8_b8_o8(x[rows], w, bias, a2, beta)
+        assert np.unique(want2).size > 200 and np.array_equal(got2[rows], want2)
+    elif which == "fc1_gelu":
+        bias = g.standard_normal(N).astype(np.float32)
+        a2 = np.float32(3.0 / (np.sqrt(K) * 127 * 127 / 3)); b2 = np.float32(20.0)
+        got = cpu(fused.linear_a8_w8_bfp32_ofp32_GeLu_Q(gx, gw, gpu(bias), a2, b2))
+        mx, rate = mismatch_report(got[rows], O.linear_a8_w8_bfp32_ofp32_GeLu_Q(x[rows], w, bias, a2, b2))
+        print(f"GELU-Q fc1: max diff {mx}, mismatch rate {rate:.2e}")
+        assert mx <= 1 and rate < 1e-3
+    else:
+        bias = g.standard_normal(N).astype(np.float32)
+        got = cpu(linear.linear_a8_w8_bfp32_ofp32(gx, gw, gpu(bias), alpha, 1.0))
+        want = O.linear_a8_w8_bfp32_ofp32(x[rows], w, bias, alpha, 1.0)
+        assert np.array_equal(got[rows], want)
+    # size-independent property over the whole output: acc(x1 + x2) == acc(x1) + acc(x2) in int32
+    x1 = rand_i8(g, M, K, lo=-60, hi=60); x2 = rand_i8(g, M, K, lo=-60, hi=60)
+    s = cpu(linear.linear_a8_w8_b32_o32(gpu((x1 + x2).astype(np.int8)), gw, None))
+    p1 = cpu(linear.linear_a8_w8_b32_o32(gpu(x1), gw, None)); p2 = cpu(linear.linear_a8_w8_b32_o32(gpu(x2), gw, None))
+    assert np.array_equal(s, p1 + p2)

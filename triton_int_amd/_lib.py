@@ -1,0 +1,117 @@
+"""ctypes binding of libtriton_int_hip.so (declared in include/triton_int_hip.h).
+
+torch is imported first on purpose: the library needs libamdhip64.so.7, and torch carries its
+own copy with that SONAME; loading torch first makes both share one HIP runtime (one context,
+interchangeable streams and device pointers).
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import torch  # noqa: F401  (must precede the CDLL below)
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libtriton_int_hip.so")
+
+# enum ti_epilogue / ti_dtype / ti_bias / ti_round
+EPI_I32, EPI_SCALE_I32, EPI_SCALE_I8, EPI_SCALE_RELU_I8, EPI_SCALE_F, EPI_GELU_I8 = range(6)
+DT_I8, DT_I32, DT_F32, DT_F16, DT_BF16 = range(5)
+BIAS_NONE, BIAS_I8, BIAS_I32, BIAS_F32 = range(4)
+ROUND_RNE_CLAMP, ROUND_TRUNC = 0, 1
+
+TORCH_TO_DT = {torch.int8: DT_I8, torch.int32: DT_I32, torch.float32: DT_F32, torch.float16: DT_F16,
+               torch.bfloat16: DT_BF16}
+TORCH_TO_BIAS = {torch.int8: BIAS_I8, torch.int32: BIAS_I32, torch.float32: BIAS_F32}
+
+EXPORTS = ("ti_version", "ti_last_error", "ti_bmm_i8", "ti_bmm_i8_config", "ti_gemm_num_configs",
+           "ti_gemm_config_name", "ti_layernorm_q", "ti_dq_add_layernorm_q", "ti_gelu_q")
+
+_lib = None
+
+_vp, _i64, _int, _f32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_float
+
+
+def _declare(lib):
+    lib.ti_version.restype = _int
+    lib.ti_version.argtypes = []
+    lib.ti_last_error.restype = ctypes.c_char_p
+    lib.ti_last_error.argtypes = []
+    bmm_args = [_vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64,
+                _int, _int, _int, _int, _vp, _int, _vp, _vp, _int, _int, _int]
+    lib.ti_bmm_i8.restype = _int
+    lib.ti_bmm_i8.argtypes = bmm_args + [_vp]
+    lib.ti_bmm_i8_config.restype = _int
+    lib.ti_bmm_i8_config.argtypes = bmm_args + [_int, _vp]
+    lib.ti_gemm_num_configs.restype = _int
+    lib.ti_gemm_num_configs.argtypes = []
+    lib.ti_gemm_config_name.restype = ctypes.c_char_p
+    lib.ti_gemm_config_name.argtypes = [_int]
+    lib.ti_layernorm_q.restype = _int
+    lib.ti_layernorm_q.argtypes = [_vp, _i64, _vp, _vp, _f32, _vp, _i64, _int, _int, _int, _int, _vp, _vp, _vp]
+    lib.ti_dq_add_layernorm_q.restype = _int
+    lib.ti_dq_add_layernorm_q.argtypes = [_vp, _i64, _f32, _vp, _i64, _vp, _vp, _f32, _vp, _i64, _vp, _i64,
+                                          _vp, _i64, _int, _int, _int, _vp, _vp, _vp]
+    lib.ti_gelu_q.restype = _int
+    lib.ti_gelu_q.argtypes = [_vp, _vp, _vp, _i64, _int, _vp]
+
+
+def lib() -> ctypes.CDLL:
+    """The loaded library.  Raises if it has not been built: there is no fallback path."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m triton_int_amd.build` "
+                "(hipcc, gfx950).  triton_int_amd has no CPU or Triton fallback.")
+        handle = ctypes.CDLL(LIB_PATH)
+        _declare(handle)
+        _lib = handle
+    return _lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc == 0:
+        return
+    msg = lib().ti_last_error().decode()
+    if rc < 0:
+        # invalid-argument codes surface like the reference's Python asserts
+        raise AssertionError(f"{what}: {msg} (status {rc})")
+    raise RuntimeError(f"{what}: {msg} (hipError {rc})")
+
+
+def ptr(t) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+def current_stream(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def require_cuda(*tensors) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError(
+                "triton_int_amd kernels run on the GPU only (got a tensor on "
+                f"{t.device}); there is no CPU fallback")
+
+
+_scalar_cache: dict = {}
+
+
+def scale_tensor(v, device) -> torch.Tensor:
+    """Scales are 0-dim fp32 device tensors read inside the kernel (the reference does
+    tl.load(scale), kernels/linear.py:227,247).  Python floats, which the reference's own
+    scripts also pass (kernels/bmm.py:777), are uploaded once and cached by value."""
+    if torch.is_tensor(v):
+        if v.device != device or v.dtype != torch.float32:
+            v = v.to(device=device, dtype=torch.float32)
+        return v
+    key = (float(v), str(device))
+    t = _scalar_cache.get(key)
+    if t is None:
+        if len(_scalar_cache) > 4096:
+            _scalar_cache.clear()
+        t = torch.tensor(float(v), dtype=torch.float32, device=device)
+        _scalar_cache[key] = t
+    return t

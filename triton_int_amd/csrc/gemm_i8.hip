@@ -1,0 +1,594 @@
+// gemm_i8.hip — int8 x int8 -> int32 GEMM / batched GEMM for gfx950 (MI355X) with fused epilogues.
+//
+// Replaces the Triton kernels of zhanglei1172/triton_int kernels/linear.py:24-853,
+// kernels/bmm.py:12-760 and kernels/fused.py:88-231 (one tl.dot K loop + per-kernel epilogue).
+//
+// Two kernel families:
+//   gemm_mfma_kernel   both operands K-contiguous and 16-byte aligned.  128-bit buffer loads
+//                      (optionally straight into LDS), XOR-swizzled LDS tiles, double buffering,
+//                      v_mfma_i32_32x32x32_i8 with a 64-lane wavefront owning a WTM x WTN sub-tile.
+//   gemm_gather_kernel any strides / alignment / K (byte gathers); same MFMA and epilogue.
+//
+// C = epilogue(sum_k A[m,k] * B[n,k]); A is [M,K], B is [N,K] (the reference's "N" operand,
+// kernels/linear.py:217), the "T" operand [K,N] arrives as strides (sBn = 1, sBk = N).
+#include "ti_common.h"
+
+namespace ti {
+
+struct GemmParams {
+  const int8_t* A;
+  const int8_t* B;
+  void* C;
+  int64_t sAb, sAm, sAk, sBb, sBn, sBk, sCb, sCm, sCn;
+  int batch, M, N, K;
+  const void* bias;
+  int bias_kind;
+  const float* alpha;
+  const float* beta;
+  int epilogue, out_dtype, round_mode;
+  int tiles_m, tiles_n, group_m;
+};
+
+enum OutClass { OUT8 = 0, OUT32 = 1, OUT16 = 2 };
+
+// ---- tile -> (m, n) mapping ----------------------------------------------------------------
+// Workgroups are dealt round-robin to the 8 XCDs (each with a private L2), so consecutive
+// block ids are first folded into 8 contiguous ranges (one per XCD) and each range then walks
+// the tile grid in column-major groups of `group_m` row-tiles so that a range re-uses few
+// distinct A and B panels.
+__device__ __forceinline__ void tile_coords(const GemmParams& p, int pid, int& tm, int& tn) {
+  const int T = p.tiles_m * p.tiles_n;
+  const int xcd = pid & 7, local = pid >> 3;
+  const int per = T >> 3, rem = T & 7;
+  const int lid = xcd * per + min(xcd, rem) + local;
+  const int gsz = p.group_m * p.tiles_n;
+  const int gid = lid / gsz;
+  const int first_m = gid * p.group_m;
+  const int gm = min(p.tiles_m - first_m, p.group_m);
+  const int r = lid - gid * gsz;
+  tm = first_m + r % gm;
+  tn = r / gm;
+}
+
+// ---- epilogue (shared by both kernel families) ------------------------------------------------
+// One fp32 value per accumulator, in the operation order the contract fixes:
+//   v = f(acc) * alpha;  c0 = f(bias) * beta;  v = c0 + v        (no FMA contraction)
+struct EpiCtx {
+  float alpha, beta;
+  int epilogue, round_mode, bias_kind;
+  const void* bias;
+};
+
+__device__ __forceinline__ float load_bias_f(const EpiCtx& e, int n) {
+  switch (e.bias_kind) {
+    case TI_BIAS_I8: return (float)((const int8_t*)e.bias)[n];
+    case TI_BIAS_I32: return (float)((const int32_t*)e.bias)[n];
+    case TI_BIAS_F32: return ((const float*)e.bias)[n];
+    default: return 0.0f;
+  }
+}
+
+// Per-column term that is added to alpha*f(acc): beta*f(bias) for the scale epilogues, the raw
+// fp32 bias for GELU-Q (kernels/fused.py:184-186 adds the bias un-scaled).
+__device__ __forceinline__ float column_term(const EpiCtx& e, int n) {
+  if (e.bias_kind == TI_BIAS_NONE) return 0.0f;
+  float b = load_bias_f(e, n);
+  return e.epilogue == TI_EPI_GELU_I8 ? b : b * e.beta;
+}
+
+__device__ __forceinline__ float epi_value(const EpiCtx& e, int acc, float col) {
+  float v = (float)acc * e.alpha;
+  if (e.bias_kind != TI_BIAS_NONE) v = col + v;
+  if (e.epilogue == TI_EPI_GELU_I8) v = gelu_tanh_scaled(v, e.beta);
+  return v;
+}
+
+__device__ __forceinline__ int epi_q8(const EpiCtx& e, int acc, float col) {
+  int q = q8(epi_value(e, acc, col), e.round_mode);
+  if (e.epilogue == TI_EPI_SCALE_RELU_I8) q = max(q, 0);
+  return q;
+}
+
+template <int OUTCLS>
+__device__ __forceinline__ void store_one(const EpiCtx& e, void* C, int64_t off, int acc, float col,
+                                          int bias_i32, int out_dtype) {
+  if constexpr (OUTCLS == OUT8) {
+    ((int8_t*)C)[off] = (int8_t)epi_q8(e, acc, col);
+  } else if constexpr (OUTCLS == OUT32) {
+    if (e.epilogue == TI_EPI_I32) {
+      ((int*)C)[off] = (int)((unsigned)acc + (unsigned)bias_i32);
+    } else if (e.epilogue == TI_EPI_SCALE_I32) {
+      ((int*)C)[off] = q32(epi_value(e, acc, col), e.round_mode);
+    } else {
+      ((float*)C)[off] = epi_value(e, acc, col);
+    }
+  } else {
+    float v = epi_value(e, acc, col);
+    ((uint16_t*)C)[off] = out_dtype == TI_F16 ? f32_to_f16_bits(v) : f32_to_bf16_bits(v);
+  }
+}
+
+__device__ __forceinline__ EpiCtx make_epi(const GemmParams& p) {
+  EpiCtx e;
+  e.alpha = p.alpha ? *p.alpha : 1.0f;
+  e.beta = p.beta ? *p.beta : 1.0f;
+  e.epilogue = p.epilogue;
+  e.round_mode = p.round_mode;
+  e.bias_kind = p.bias ? p.bias_kind : TI_BIAS_NONE;
+  e.bias = p.bias;
+  return e;
+}
+
+// ---- fast family -----------------------------------------------------------------------------
+//
+// LDS tile = ROWS x BK bytes, viewed as 16-byte chunks; chunk c of row r lives at chunk slot
+// c ^ ((r >> SWZ) & (CH-1)) of that row, which spreads the 16-byte reads of the 32 lanes that
+// share a chunk index (one MFMA operand column) over the banks.
+//
+// Loads: chunk slot q = it*NT + tid of the tile is filled by thread tid.  LOADMODE 0 goes
+// through registers (buffer_load_dwordx4 + ds_write_b128); LOADMODE 1 lets the buffer load write
+// LDS itself (buffer_load_dwordx4 ... lds: lane i of a wave lands at M0-base + 16*i).
+// Buffer descriptors bound the loads: rows past M/N and the K tail read as zero.
+
+template <int ROWS, int BK, int NT, int SWZ>
+struct TileLoader {
+  static constexpr int CH = BK / 16;
+  static constexpr int IT = ROWS * CH / NT;
+  static_assert(ROWS * CH % NT == 0, "tile must split evenly over the threads");
+  int voff[IT];  // byte offset of the chunk at k-tile 0; advanced by BK per k-tile
+  int kpos[IT];  // k index of the chunk at k-tile 0
+
+  __device__ __forceinline__ void init(int tid, int row0, int ld) {
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+      const int q = it * NT + tid;
+      const int row = q / CH;
+      const int cphys = q % CH;
+      const int clog = cphys ^ ((row >> SWZ) & (CH - 1));
+      voff[it] = (row0 + row) * ld + clog * 16;
+      kpos[it] = clog * 16;
+    }
+  }
+};
+
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int SWZ, int LOADMODE, int OUTCLS>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmParams p) {
+  constexpr int NT = WAVES_M * WAVES_N * 64;
+  constexpr int CH = BK / 16;
+  constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int KS = BK / 32;  // MFMA k-steps per k-tile
+  constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
+  constexpr int STAGE = A_BYTES + B_BYTES;
+  constexpr int C_PITCH = BN + 4;  // int8 staging pitch: 33-dword rows keep dword writes conflict-free
+  constexpr int LDS_BYTES = (2 * STAGE > BM * C_PITCH) ? 2 * STAGE : BM * C_PITCH;
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % 32 == 0, "tile shape");
+
+  __shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+  int tile_m, tile_n;
+  tile_coords(p, blockIdx.x, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int bz = blockIdx.y;
+
+  const int8_t* Ab = p.A + (int64_t)bz * p.sAb;
+  const int8_t* Bb = p.B + (int64_t)bz * p.sBb;
+  const int lda = (int)p.sAm, ldb = (int)p.sBn;
+  // bytes addressable from the batch base: rows past the end and the K tail read as zero
+  const int a_extent = (p.M - 1) * lda + p.K;
+  const int b_extent = (p.N - 1) * ldb + p.K;
+  __amdgpu_buffer_rsrc_t rA = __builtin_amdgcn_make_buffer_rsrc((void*)Ab, 0, a_extent, 0x00020000);
+  __amdgpu_buffer_rsrc_t rB = __builtin_amdgcn_make_buffer_rsrc((void*)Bb, 0, b_extent, 0x00020000);
+
+  TileLoader<BM, BK, NT, SWZ> la;
+  TileLoader<BN, BK, NT, SWZ> lb;
+  la.init(tid, m0, lda);
+  lb.init(tid, n0, ldb);
+  constexpr int A_IT = decltype(la)::IT, B_IT = decltype(lb)::IT;
+  const int KT = (p.K + BK - 1) / BK;
+  const int OOB = (int)0x80000000;
+
+  v4u ra[LOADMODE == 0 ? A_IT : 1], rb[LOADMODE == 0 ? B_IT : 1];
+
+  // issue the loads of k-tile kt (into registers, or straight into LDS stage `st`)
+  auto issue = [&](int kt, int st) {
+    const int k0 = kt * BK;
+    char* sA = lds + st * STAGE;
+    char* sB = sA + A_BYTES;
+#pragma unroll
+    for (int it = 0; it < A_IT; ++it) {
+      const int vo = (k0 + la.kpos[it] < p.K) ? la.voff[it] + k0 : OOB;
+      if constexpr (LOADMODE == 0) {
+        ra[it] = __builtin_amdgcn_raw_buffer_load_b128(rA, vo, 0, 0);
+      } else {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rA, (void __attribute__((address_space(3)))*)(sA + (it * NT + wave * 64) * 16), 16, vo, 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < B_IT; ++it) {
+      const int vo = (k0 + lb.kpos[it] < p.K) ? lb.voff[it] + k0 : OOB;
+      if constexpr (LOADMODE == 0) {
+        rb[it] = __builtin_amdgcn_raw_buffer_load_b128(rB, vo, 0, 0);
+      } else {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rB, (void __attribute__((address_space(3)))*)(sB + (it * NT + wave * 64) * 16), 16, vo, 0, 0, 0);
+      }
+    }
+  };
+  // LOADMODE 0 only: registers -> LDS stage st
+  auto commit = [&](int st) {
+    if constexpr (LOADMODE == 0) {
+      char* sA = lds + st * STAGE;
+      char* sB = sA + A_BYTES;
+#pragma unroll
+      for (int it = 0; it < A_IT; ++it) *(v4u*)(sA + (it * NT + tid) * 16) = ra[it];
+#pragma unroll
+      for (int it = 0; it < B_IT; ++it) *(v4u*)(sB + (it * NT + tid) * 16) = rb[it];
+    }
+  };
+
+  v16i acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+  // per-lane fragment addressing: row = (lane & 31) within a 32-row MFMA operand block,
+  // logical chunk = 2*ks + (lane >> 5)
+  const int frow = lane & 31;
+  const int fsw = (frow >> SWZ) & (CH - 1);
+  const int fhalf = lane >> 5;
+  const int a_lane = (wm * WTM + frow) * BK;
+  const int b_lane = (wn * WTN + frow) * BK;
+
+  if (KT > 0) {
+    issue(0, 0);
+    if constexpr (LOADMODE == 0) commit(0);
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  }
+
+  for (int kt = 0; kt < KT; ++kt) {
+    const int st = kt & 1;
+    if (kt + 1 < KT) issue(kt + 1, st ^ 1);
+    const char* sA = lds + st * STAGE;
+    const char* sB = sA + A_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int coff = ((ks * 2 + fhalf) ^ fsw) * 16;
+      v4i fa[TM], fb[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) fa[i] = *(const v4i*)(sA + a_lane + i * 32 * BK + coff);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) fb[j] = *(const v4i*)(sB + b_lane + j * 32 * BK + coff);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          if constexpr (OUTCLS == OUT8)  // rows of the MFMA result = n (4 consecutive n per lane)
+            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[j], fa[i], acc[i][j], 0, 0, 0);
+          else  // rows of the MFMA result = m, lanes run along n
+            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+    }
+    if (kt + 1 < KT) {
+      if constexpr (LOADMODE == 0) commit(st ^ 1);
+      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue ----
+  const EpiCtx e = make_epi(p);
+  char* Cb = (char*)p.C;
+  const int lrow = lane & 31, lhi = lane >> 5;
+
+  if constexpr (OUTCLS == OUT8) {
+    // acc[i][j][r]: m = m0 + wm*WTM + i*32 + lrow;  n = n0 + wn*WTN + j*32 + 8*(r/4) + 4*lhi + r%4.
+    // Quantise, pack 4 consecutive n into a dword, stage the tile in LDS, then write rows with
+    // 16-byte stores.  (The K loop ended with a barrier, so the operand stages are free.)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int nl = wn * WTN + j * 32 + 8 * g + 4 * lhi;
+        float col[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) col[t] = column_term(e, min(n0 + nl + t, p.N - 1));
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          const int ml = wm * WTM + i * 32 + lrow;
+          const unsigned w = pack4(epi_q8(e, acc[i][j][4 * g + 0], col[0]), epi_q8(e, acc[i][j][4 * g + 1], col[1]),
+                                   epi_q8(e, acc[i][j][4 * g + 2], col[2]), epi_q8(e, acc[i][j][4 * g + 3], col[3]));
+          *(unsigned*)(lds + ml * C_PITCH + nl) = w;
+        }
+      }
+    }
+    __syncthreads();
+    int8_t* Cz = (int8_t*)Cb + (int64_t)bz * p.sCb;
+    const bool vec_ok = ((p.sCm & 15) == 0) && ((((uintptr_t)Cz) & 15) == 0);
+    constexpr int SEGS = BN / 16;
+    for (int s = tid; s < BM * SEGS; s += NT) {
+      const int ml = s / SEGS, seg = s % SEGS;
+      const int m = m0 + ml, n = n0 + seg * 16;
+      if (m >= p.M || n >= p.N) continue;
+      const unsigned* src = (const unsigned*)(lds + ml * C_PITCH + seg * 16);
+      v4u v;
+      v[0] = src[0]; v[1] = src[1]; v[2] = src[2]; v[3] = src[3];
+      int8_t* dst = Cz + (int64_t)m * p.sCm + n;
+      if (vec_ok && n + 16 <= p.N) {
+        *(v4u*)dst = v;
+      } else {
+        const int cnt = min(16, p.N - n);
+        for (int t = 0; t < cnt; ++t) dst[t] = (int8_t)(v[t >> 2] >> ((t & 3) * 8));
+      }
+    }
+  } else {
+    // acc[i][j][r]: m = m0 + wm*WTM + i*32 + 8*(r/4) + 4*lhi + r%4;  n = n0 + wn*WTN + j*32 + lrow.
+    constexpr int ESZ = OUTCLS == OUT32 ? 4 : 2;
+    char* Cz = Cb + (int64_t)bz * p.sCb * ESZ;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int n = n0 + wn * WTN + j * 32 + lrow;
+      const int nc = min(n, p.N - 1);
+      const float col = column_term(e, nc);
+      const int bias_i32 = (e.epilogue == TI_EPI_I32 && e.bias_kind == TI_BIAS_I32) ? ((const int*)e.bias)[nc] : 0;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = m0 + wm * WTM + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+          if (m < p.M && n < p.N)
+            store_one<OUTCLS>(e, Cz, (int64_t)m * p.sCm + (int64_t)n * p.sCn, acc[i][j][r], col, bias_i32, p.out_dtype);
+        }
+      }
+    }
+  }
+}
+
+// ---- gather family -----------------------------------------------------------------------------
+// 64x64 tile, BK = 32, 4 waves each owning one 32x32 MFMA block.  Every byte is fetched on its
+// own with 64-bit addressing, so any stride pattern, alignment and K works.
+template <int OUTCLS>
+__global__ __launch_bounds__(256) void gemm_gather_kernel(GemmParams p) {
+  constexpr int BM = 64, BN = 64, BK = 32, PITCH = BK + 16;  // 48-byte rows: 16-byte aligned, de-phased banks
+  __shared__ __attribute__((aligned(16))) char sA[BM * PITCH];
+  __shared__ __attribute__((aligned(16))) char sB[BN * PITCH];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  int tile_m, tile_n;
+  tile_coords(p, blockIdx.x, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN, bz = blockIdx.y;
+  const int8_t* Ab = p.A + (int64_t)bz * p.sAb;
+  const int8_t* Bb = p.B + (int64_t)bz * p.sBb;
+  // walk the tile so that consecutive threads touch consecutive memory when a unit stride exists
+  const bool a_kfast = p.sAk == 1 || p.sAm != 1;
+  const bool b_kfast = p.sBk == 1 || p.sBn != 1;
+
+  v16i acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0;
+
+  const int KT = (p.K + BK - 1) / BK;
+  for (int kt = 0; kt < KT; ++kt) {
+    const int k0 = kt * BK;
+#pragma unroll
+    for (int it = 0; it < BM * BK / 256; ++it) {
+      const int e = it * 256 + tid;
+      const int r = a_kfast ? e / BK : e % BM;
+      const int k = a_kfast ? e % BK : e / BM;
+      int8_t v = 0;
+      if (m0 + r < p.M && k0 + k < p.K) v = Ab[(int64_t)(m0 + r) * p.sAm + (int64_t)(k0 + k) * p.sAk];
+      sA[r * PITCH + k] = v;
+    }
+#pragma unroll
+    for (int it = 0; it < BN * BK / 256; ++it) {
+      const int e = it * 256 + tid;
+      const int r = b_kfast ? e / BK : e % BN;
+      const int k = b_kfast ? e % BK : e / BN;
+      int8_t v = 0;
+      if (n0 + r < p.N && k0 + k < p.K) v = Bb[(int64_t)(n0 + r) * p.sBn + (int64_t)(k0 + k) * p.sBk];
+      sB[r * PITCH + k] = v;
+    }
+    __syncthreads();
+    const v4i fa = *(const v4i*)(sA + (wm * 32 + (lane & 31)) * PITCH + (lane >> 5) * 16);
+    const v4i fb = *(const v4i*)(sB + (wn * 32 + (lane & 31)) * PITCH + (lane >> 5) * 16);
+    acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa, fb, acc, 0, 0, 0);
+    __syncthreads();
+  }
+
+  const EpiCtx e = make_epi(p);
+  constexpr int ESZ = OUTCLS == OUT8 ? 1 : (OUTCLS == OUT32 ? 4 : 2);
+  char* Cz = (char*)p.C + (int64_t)bz * p.sCb * ESZ;
+  const int n = n0 + wn * 32 + (lane & 31);
+  const int nc = min(n, p.N - 1);
+  const float col = column_term(e, nc);
+  const int bias_i32 = (e.epilogue == TI_EPI_I32 && e.bias_kind == TI_BIAS_I32) ? ((const int*)e.bias)[nc] : 0;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int m = m0 + wm * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+    if (m < p.M && n < p.N)
+      store_one<OUTCLS>(e, Cz, (int64_t)m * p.sCm + (int64_t)n * p.sCn, acc[r], col, bias_i32, p.out_dtype);
+  }
+}
+
+// ---- host side ---------------------------------------------------------------------------------
+
+typedef void (*KernelFn)(GemmParams);
+
+struct Config {
+  const char* name;
+  KernelFn fn[3];  // by OutClass
+  int bm, bn, bk, threads;
+  bool fast;       // needs the aligned K-contiguous layout
+};
+
+#define TI_FAST(BM, BN, BK, WM, WN, SWZ, LM)                                              \
+  {                                                                                       \
+    "mfma_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN "_s" #SWZ "_l" #LM,                        \
+        {gemm_mfma_kernel<BM, BN, BK, WM, WN, SWZ, LM, OUT8>,                               \
+         gemm_mfma_kernel<BM, BN, BK, WM, WN, SWZ, LM, OUT32>,                              \
+         gemm_mfma_kernel<BM, BN, BK, WM, WN, SWZ, LM, OUT16>},                             \
+        BM, BN, BK, WM * WN * 64, true                                                    \
+  }
+
+static const Config g_configs[] = {
+    {"gather_64x64x32", {gemm_gather_kernel<OUT8>, gemm_gather_kernel<OUT32>, gemm_gather_kernel<OUT16>}, 64, 64, 32, 256, false},
+    TI_FAST(256, 128, 128, 2, 2, 0, 0),
+    TI_FAST(256, 128, 128, 2, 2, 0, 1),
+    TI_FAST(256, 128, 128, 2, 2, 1, 1),
+    TI_FAST(128, 128, 128, 2, 2, 0, 0),
+    TI_FAST(128, 128, 128, 2, 2, 0, 1),
+    TI_FAST(256, 128, 64, 2, 2, 1, 0),
+    TI_FAST(256, 128, 64, 2, 2, 1, 1),
+    TI_FAST(256, 128, 64, 2, 2, 2, 1),
+    TI_FAST(128, 256, 128, 2, 2, 0, 1),
+    TI_FAST(64, 64, 128, 2, 2, 0, 1),
+};
+static const int g_num_configs = (int)(sizeof(g_configs) / sizeof(g_configs[0]));
+
+static int out_class(int out_dtype) {
+  switch (out_dtype) {
+    case TI_I8: return OUT8;
+    case TI_I32:
+    case TI_F32: return OUT32;
+    default: return OUT16;
+  }
+}
+
+static bool fast_eligible(const GemmParams& p) {
+  if (p.sAk != 1 || p.sBk != 1) return false;
+  if (p.K <= 0 || (p.K & 15)) return false;
+  if ((p.sAm & 15) || (p.sBn & 15) || (p.sAb & 15) || (p.sBb & 15)) return false;
+  if (((uintptr_t)p.A & 15) || ((uintptr_t)p.B & 15)) return false;
+  if (p.sAm < p.K || p.sBn < p.K) return false;
+  if (out_class(p.out_dtype) == OUT8 && p.sCn != 1) return false;
+  // 32-bit byte offsets inside one batch slice, including the rows a ragged last tile touches
+  const int64_t lim = (int64_t)1 << 31;
+  if (((int64_t)p.M + 256) * p.sAm + p.K >= lim) return false;
+  if (((int64_t)p.N + 256) * p.sBn + p.K >= lim) return false;
+  return true;
+}
+
+static int pick_config(const GemmParams& p) {
+  if (!fast_eligible(p)) return 0;
+  // Largest tile that still gives every CU work; measured preferences are encoded as the
+  // candidate order.
+  const int64_t cus = 256;
+  const int cand[] = {2, 5, 10};
+  for (int c : cand) {
+    const Config& k = g_configs[c];
+    const int64_t tiles = (int64_t)((p.M + k.bm - 1) / k.bm) * ((p.N + k.bn - 1) / k.bn) * p.batch;
+    if (tiles >= cus || c == 10) return c;
+  }
+  return 10;
+}
+
+static int pick_group_m(const GemmParams& p, const Config& k) {
+  // each XCD runs tiles/8 consecutive tiles; make that range roughly square in rows touched
+  const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
+  const int per_xcd = (int)((tiles + 7) / 8);
+  int best = 1;
+  int64_t best_cost = -1;
+  for (int g = 1; g <= p.tiles_m && g <= 64; g *= 2) {
+    const int cols = (per_xcd + g - 1) / g;
+    const int64_t cost = (int64_t)g * k.bm + (int64_t)cols * k.bn;
+    if (best_cost < 0 || cost < best_cost) best_cost = cost, best = g;
+  }
+  return best;
+}
+
+static int validate(const GemmParams& p) {
+  if (p.batch < 0 || p.M < 0 || p.N < 0 || p.K < 0) return fail(TI_E_SHAPE, "negative size");
+  if (p.batch == 0 || p.M == 0 || p.N == 0) return TI_OK;
+  if (!p.A && p.K > 0) return fail(TI_E_NULL, "A is NULL");
+  if (!p.B && p.K > 0) return fail(TI_E_NULL, "B is NULL");
+  if (!p.C) return fail(TI_E_NULL, "C is NULL");
+  if (p.batch > 65535) return fail(TI_E_SHAPE, "batch %d > 65535", p.batch);
+  const int bk = p.bias ? p.bias_kind : TI_BIAS_NONE;
+  bool ok = false;
+  switch (p.epilogue) {
+    case TI_EPI_I32: ok = p.out_dtype == TI_I32 && (bk == TI_BIAS_NONE || bk == TI_BIAS_I32); break;
+    case TI_EPI_SCALE_I32: ok = p.out_dtype == TI_I32 && (bk == TI_BIAS_NONE || bk == TI_BIAS_I32); break;
+    case TI_EPI_SCALE_I8:
+    case TI_EPI_SCALE_RELU_I8: ok = p.out_dtype == TI_I8 && (bk == TI_BIAS_NONE || bk == TI_BIAS_I8); break;
+    case TI_EPI_SCALE_F:
+      ok = (p.out_dtype == TI_F32 || p.out_dtype == TI_F16 || p.out_dtype == TI_BF16) && (bk == TI_BIAS_NONE || bk == TI_BIAS_F32);
+      break;
+    case TI_EPI_GELU_I8: ok = p.out_dtype == TI_I8 && (bk == TI_BIAS_NONE || bk == TI_BIAS_F32); break;
+    default: break;
+  }
+  if (!ok) return fail(TI_E_COMBO, "epilogue %d / out dtype %d / bias kind %d is not a defined combination", p.epilogue, p.out_dtype, bk);
+  if (p.epilogue != TI_EPI_I32 && !p.alpha) return fail(TI_E_NULL, "alpha is NULL");
+  if (bk != TI_BIAS_NONE && p.epilogue != TI_EPI_I32 && !p.beta) return fail(TI_E_NULL, "beta is NULL");
+  if (p.epilogue == TI_EPI_GELU_I8 && !p.beta) return fail(TI_E_NULL, "beta (output scale) is NULL");
+  if (p.round_mode != TI_ROUND_RNE_CLAMP && p.round_mode != TI_ROUND_TRUNC) return fail(TI_E_COMBO, "round mode %d", p.round_mode);
+  if (p.sCm == 0 && p.M > 1) return fail(TI_E_STRIDE, "output row stride is 0");
+  if (p.sCn == 0 && p.N > 1) return fail(TI_E_STRIDE, "output column stride is 0");
+  return TI_OK;
+}
+
+static int run(GemmParams p, int config, hipStream_t stream) {
+  int rc = validate(p);
+  if (rc != TI_OK) return rc;
+  if (p.batch == 0 || p.M == 0 || p.N == 0) return TI_OK;
+  rc = check_device();
+  if (rc != TI_OK) return rc;
+  if (!p.bias) p.bias_kind = TI_BIAS_NONE;
+  if (config < 0) config = pick_config(p);
+  if (config >= g_num_configs) return fail(TI_E_COMBO, "config %d out of range", config);
+  const Config& k = g_configs[config];
+  if (k.fast && !fast_eligible(p)) return fail(TI_E_COMBO, "config %s needs K-contiguous 16-byte aligned operands", k.name);
+  p.tiles_m = (p.M + k.bm - 1) / k.bm;
+  p.tiles_n = (p.N + k.bn - 1) / k.bn;
+  if ((int64_t)p.tiles_m * p.tiles_n > 0x7fffffff) return fail(TI_E_SHAPE, "too many tiles");
+  p.group_m = pick_group_m(p, k);
+  dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)p.batch, 1);
+  k.fn[out_class(p.out_dtype)]<<<grid, dim3(k.threads), 0, stream>>>(p);
+  return launch_status(k.name);
+}
+
+}  // namespace ti
+
+extern "C" {
+
+int ti_bmm_i8_config(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk, const int8_t* B, int64_t sBb,
+                     int64_t sBn, int64_t sBk, void* C, int64_t sCb, int64_t sCm, int64_t sCn, int batch, int M,
+                     int N, int K, const void* bias, int bias_kind, const float* alpha, const float* beta,
+                     int epilogue, int out_dtype, int round_mode, int config, void* stream) {
+  ti::GemmParams p;
+  p.A = A; p.B = B; p.C = C;
+  p.sAb = sAb; p.sAm = sAm; p.sAk = sAk;
+  p.sBb = sBb; p.sBn = sBn; p.sBk = sBk;
+  p.sCb = sCb; p.sCm = sCm; p.sCn = sCn;
+  p.batch = batch; p.M = M; p.N = N; p.K = K;
+  p.bias = bias; p.bias_kind = bias_kind;
+  p.alpha = alpha; p.beta = beta;
+  p.epilogue = epilogue; p.out_dtype = out_dtype; p.round_mode = round_mode;
+  p.tiles_m = p.tiles_n = 0; p.group_m = 1;
+  return ti::run(p, config, (hipStream_t)stream);
+}
+
+int ti_bmm_i8(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk, const int8_t* B, int64_t sBb, int64_t sBn,
+              int64_t sBk, void* C, int64_t sCb, int64_t sCm, int64_t sCn, int batch, int M, int N, int K,
+              const void* bias, int bias_kind, const float* alpha, const float* beta, int epilogue, int out_dtype,
+              int round_mode, void* stream) {
+  return ti_bmm_i8_config(A, sAb, sAm, sAk, B, sBb, sBn, sBk, C, sCb, sCm, sCn, batch, M, N, K, bias, bias_kind,
+                          alpha, beta, epilogue, out_dtype, round_mode, -1, stream);
+}
+
+int ti_gemm_num_configs(void) { return ti::g_num_configs; }
+
+const char* ti_gemm_config_name(int config) {
+  return (config >= 0 && config < ti::g_num_configs) ? ti::g_configs[config].name : "";
+}
+
+}  // extern "C"

@@ -1,0 +1,326 @@
+// rowops.hip — HBM-bound row kernels for gfx950: LayerNorm -> int8, dequant + residual add +
+// LayerNorm -> int8, and tanh-GELU -> int8.
+//
+// Replaces kernel_layer_norm_fwd_fused_single_pass_q (kernels/fused.py:235-382 of
+// zhanglei1172/triton_int), supplies the native dq_add_layernorm_q the reference only emulates
+// (functional/fused.py:6-32) and a launchable form of fast_geluQ (kernels/fused.py:76-79).
+//
+// Row kernels: one row per 256-thread workgroup.  The whole row sits in registers as float4
+// vectors (thread t owns vectors t, t+256, ...: every load/store instruction of a wave is one
+// contiguous 1 KB / 256 B run), so x is read from HBM exactly once; mean and the centred sum of
+// squares are exact two-pass statistics reduced with wave shuffles and one LDS hop.
+#include "ti_common.h"
+
+namespace ti {
+
+constexpr int RN_THREADS = 256;
+constexpr int RN_WAVES = RN_THREADS / 64;
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+// Sum over the workgroup; every thread returns the same bits (fixed combination order).
+__device__ __forceinline__ float block_sum(float v, float* red, int tid) {
+  v = wave_sum(v);
+  __syncthreads();  // protect `red` from the previous use
+  if ((tid & 63) == 0) red[tid >> 6] = v;
+  __syncthreads();
+  float s = red[0];
+#pragma unroll
+  for (int w = 1; w < RN_WAVES; ++w) s += red[w];
+  return s;
+}
+
+struct RowNormParams {
+  const float* x;        // LN input (DQ = false)
+  const int32_t* acc;    // DQ: int32 accumulator
+  const float* resid_in; // DQ
+  float* resid_out;      // DQ
+  int64_t x_rs, acc_rs, rin_rs, rout_rs, y_rs, ln_rs;
+  float in_scale;
+  const float* gamma;
+  const float* beta;
+  float eps;
+  int8_t* y;
+  float* ln_out;
+  float* mean_out;
+  float* rstd_out;
+  int rows, cols, rms, round_mode;
+};
+
+__device__ __forceinline__ float norm_one(float x, float mean, float rstd, float w, float b, bool has_b) {
+  // kernels/fused.py:323-327: a_hat = (a - mean) * rstd; out = a_hat * weight (+ bias)
+  float o = ((x - mean) * rstd) * w;
+  return has_b ? o + b : o;
+}
+
+template <int VPT, bool DQ>
+__global__ __launch_bounds__(RN_THREADS) void rownorm_vec_kernel(RowNormParams p) {
+  __shared__ float red[RN_WAVES];
+  const int tid = threadIdx.x;
+  const int row = blockIdx.x;
+  const int nvec = p.cols >> 2;
+
+  v4f x[VPT];
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int v = tid + j * RN_THREADS;
+    if (v < nvec) {
+      if constexpr (DQ) {
+        const v4i a = *(const v4i*)(p.acc + (int64_t)row * p.acc_rs + v * 4);
+        const v4f r = *(const v4f*)(p.resid_in + (int64_t)row * p.rin_rs + v * 4);
+        v4f o;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          // functional/fused.py:9: residual + alpha * int32 (product and sum rounded separately)
+          const float prod = p.in_scale * (float)a[t];
+          o[t] = r[t] + prod;
+        }
+        x[j] = o;
+        *(v4f*)(p.resid_out + (int64_t)row * p.rout_rs + v * 4) = o;
+      } else {
+        x[j] = *(const v4f*)(p.x + (int64_t)row * p.x_rs + v * 4);
+      }
+    } else {
+      x[j] = (v4f){0.f, 0.f, 0.f, 0.f};
+    }
+  }
+
+  const float inv_n = 1.0f / (float)p.cols;
+  float mean = 0.0f;
+  if (!p.rms) {
+    float s = 0.0f;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) s += (x[j][0] + x[j][1]) + (x[j][2] + x[j][3]);
+    mean = block_sum(s, red, tid) * inv_n;
+  }
+  float m2 = 0.0f;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int v = tid + j * RN_THREADS;
+    if (v < nvec) {
+      const float d0 = x[j][0] - mean, d1 = x[j][1] - mean, d2 = x[j][2] - mean, d3 = x[j][3] - mean;
+      m2 += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
+    }
+  }
+  const float var = block_sum(m2, red, tid) * inv_n;
+  const float rstd = 1.0f / sqrtf(var + p.eps);
+  if (tid == 0) {
+    if (p.mean_out) p.mean_out[row] = mean;
+    if (p.rstd_out) p.rstd_out[row] = rstd;
+  }
+
+  const bool has_b = p.beta != nullptr;
+  const bool y_vec = p.y && ((p.y_rs & 3) == 0) && ((((uintptr_t)p.y) & 3) == 0);
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int v = tid + j * RN_THREADS;
+    if (v < nvec) {
+      const v4f w = *(const v4f*)(p.gamma + v * 4);
+      v4f b = {0.f, 0.f, 0.f, 0.f};
+      if (has_b) b = *(const v4f*)(p.beta + v * 4);
+      v4f o;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) o[t] = norm_one(x[j][t], mean, rstd, w[t], b[t], has_b);
+      if (p.ln_out) *(v4f*)(p.ln_out + (int64_t)row * p.ln_rs + v * 4) = o;
+      if (p.y) {
+        const int q0 = q8(o[0], p.round_mode), q1 = q8(o[1], p.round_mode), q2 = q8(o[2], p.round_mode),
+                  q3 = q8(o[3], p.round_mode);
+        int8_t* dst = p.y + (int64_t)row * p.y_rs + v * 4;
+        if (y_vec) {
+          *(unsigned*)dst = pack4(q0, q1, q2, q3);
+        } else {
+          dst[0] = (int8_t)q0; dst[1] = (int8_t)q1; dst[2] = (int8_t)q2; dst[3] = (int8_t)q3;
+        }
+      }
+    }
+  }
+}
+
+// Any column count / alignment: the row is re-read from memory for each pass (it stays in L2).
+template <bool DQ>
+__global__ __launch_bounds__(RN_THREADS) void rownorm_any_kernel(RowNormParams p) {
+  __shared__ float red[RN_WAVES];
+  const int tid = threadIdx.x;
+  const int row = blockIdx.x;
+  const float* xr;
+  if constexpr (DQ) {
+    const int32_t* ar = p.acc + (int64_t)row * p.acc_rs;
+    const float* rin = p.resid_in + (int64_t)row * p.rin_rs;
+    float* rout = p.resid_out + (int64_t)row * p.rout_rs;
+    for (int i = tid; i < p.cols; i += RN_THREADS) {
+      const float prod = p.in_scale * (float)ar[i];
+      rout[i] = rin[i] + prod;
+    }
+    __threadfence_block();
+    __syncthreads();
+    xr = rout;
+  } else {
+    xr = p.x + (int64_t)row * p.x_rs;
+  }
+  const float inv_n = 1.0f / (float)p.cols;
+  float mean = 0.0f;
+  if (!p.rms) {
+    float s = 0.0f;
+    for (int i = tid; i < p.cols; i += RN_THREADS) s += xr[i];
+    mean = block_sum(s, red, tid) * inv_n;
+  }
+  float m2 = 0.0f;
+  for (int i = tid; i < p.cols; i += RN_THREADS) {
+    const float d = xr[i] - mean;
+    m2 += d * d;
+  }
+  const float var = block_sum(m2, red, tid) * inv_n;
+  const float rstd = 1.0f / sqrtf(var + p.eps);
+  if (tid == 0) {
+    if (p.mean_out) p.mean_out[row] = mean;
+    if (p.rstd_out) p.rstd_out[row] = rstd;
+  }
+  const bool has_b = p.beta != nullptr;
+  for (int i = tid; i < p.cols; i += RN_THREADS) {
+    const float o = norm_one(xr[i], mean, rstd, p.gamma[i], has_b ? p.beta[i] : 0.0f, has_b);
+    if (p.ln_out) p.ln_out[(int64_t)row * p.ln_rs + i] = o;
+    if (p.y) p.y[(int64_t)row * p.y_rs + i] = (int8_t)q8(o, p.round_mode);
+  }
+}
+
+static bool aligned16(const void* ptr, int64_t row_stride_elems, int elem) {
+  return (((uintptr_t)ptr) & 15) == 0 && ((row_stride_elems * elem) & 15) == 0;
+}
+
+template <bool DQ>
+static int launch_rownorm(const RowNormParams& p, hipStream_t stream) {
+  if (p.rows == 0 || p.cols == 0) return TI_OK;
+  int rc = check_device();
+  if (rc != TI_OK) return rc;
+  bool vec = (p.cols & 3) == 0 && p.cols <= RN_THREADS * 4 * 8 && aligned16(p.gamma, 0, 4) &&
+             (!p.beta || aligned16(p.beta, 0, 4)) && (!p.ln_out || aligned16(p.ln_out, p.ln_rs, 4));
+  if (DQ) vec = vec && aligned16(p.acc, p.acc_rs, 4) && aligned16(p.resid_in, p.rin_rs, 4) && aligned16(p.resid_out, p.rout_rs, 4);
+  else vec = vec && aligned16(p.x, p.x_rs, 4);
+  dim3 grid((unsigned)p.rows), block(RN_THREADS);
+  if (!vec) {
+    rownorm_any_kernel<DQ><<<grid, block, 0, stream>>>(p);
+    return launch_status("rownorm_any_kernel");
+  }
+  const int vpt = (p.cols / 4 + RN_THREADS - 1) / RN_THREADS;
+  if (vpt <= 1) rownorm_vec_kernel<1, DQ><<<grid, block, 0, stream>>>(p);
+  else if (vpt <= 2) rownorm_vec_kernel<2, DQ><<<grid, block, 0, stream>>>(p);
+  else if (vpt <= 3) rownorm_vec_kernel<3, DQ><<<grid, block, 0, stream>>>(p);
+  else if (vpt <= 4) rownorm_vec_kernel<4, DQ><<<grid, block, 0, stream>>>(p);
+  else if (vpt <= 5) rownorm_vec_kernel<5, DQ><<<grid, block, 0, stream>>>(p);
+  else if (vpt <= 6) rownorm_vec_kernel<6, DQ><<<grid, block, 0, stream>>>(p);
+  else rownorm_vec_kernel<8, DQ><<<grid, block, 0, stream>>>(p);
+  return launch_status("rownorm_vec_kernel");
+}
+
+// ---- GELU -> int8 ---------------------------------------------------------------------------
+
+constexpr int GQ_THREADS = 256;
+constexpr int GQ_UNROLL = 4;
+
+__global__ __launch_bounds__(GQ_THREADS) void gelu_q_vec_kernel(const float* __restrict__ x, const float* scale,
+                                                                int8_t* __restrict__ y, int64_t nvec,
+                                                                int round_mode) {
+  const float s = *scale;
+  const int64_t stride = (int64_t)gridDim.x * GQ_THREADS;
+  int64_t v = (int64_t)blockIdx.x * GQ_THREADS + threadIdx.x;
+  for (; v + (GQ_UNROLL - 1) * stride < nvec; v += GQ_UNROLL * stride) {
+    v4f in[GQ_UNROLL];
+#pragma unroll
+    for (int u = 0; u < GQ_UNROLL; ++u) in[u] = *(const v4f*)(x + (v + u * stride) * 4);
+#pragma unroll
+    for (int u = 0; u < GQ_UNROLL; ++u) {
+      const unsigned w = pack4(q8(gelu_tanh_scaled(in[u][0], s), round_mode), q8(gelu_tanh_scaled(in[u][1], s), round_mode),
+                               q8(gelu_tanh_scaled(in[u][2], s), round_mode), q8(gelu_tanh_scaled(in[u][3], s), round_mode));
+      *(unsigned*)(y + (v + u * stride) * 4) = w;
+    }
+  }
+  for (; v < nvec; v += stride) {
+    const v4f in = *(const v4f*)(x + v * 4);
+    const unsigned w = pack4(q8(gelu_tanh_scaled(in[0], s), round_mode), q8(gelu_tanh_scaled(in[1], s), round_mode),
+                             q8(gelu_tanh_scaled(in[2], s), round_mode), q8(gelu_tanh_scaled(in[3], s), round_mode));
+    *(unsigned*)(y + v * 4) = w;
+  }
+}
+
+__global__ __launch_bounds__(GQ_THREADS) void gelu_q_any_kernel(const float* x, const float* scale, int8_t* y,
+                                                                int64_t start, int64_t n, int round_mode) {
+  const float s = *scale;
+  const int64_t stride = (int64_t)gridDim.x * GQ_THREADS;
+  for (int64_t i = start + (int64_t)blockIdx.x * GQ_THREADS + threadIdx.x; i < n; i += stride)
+    y[i] = (int8_t)q8(gelu_tanh_scaled(x[i], s), round_mode);
+}
+
+}  // namespace ti
+
+extern "C" {
+
+int ti_layernorm_q(const float* x, int64_t x_row_stride, const float* gamma, const float* beta, float eps,
+                   int8_t* y, int64_t y_row_stride, int rows, int cols, int rms, int round_mode, float* mean_out,
+                   float* rstd_out, void* stream) {
+  if (rows < 0 || cols < 0) return ti::fail(TI_E_SHAPE, "negative size");
+  if (rows == 0 || cols == 0) return TI_OK;
+  if (!x || !gamma || !y) return ti::fail(TI_E_NULL, "x, gamma and y are required");
+  if (round_mode != TI_ROUND_RNE_CLAMP && round_mode != TI_ROUND_TRUNC) return ti::fail(TI_E_COMBO, "round mode %d", round_mode);
+  ti::RowNormParams p = {};
+  p.x = x; p.x_rs = x_row_stride;
+  p.gamma = gamma; p.beta = beta; p.eps = eps;
+  p.y = y; p.y_rs = y_row_stride;
+  p.rows = rows; p.cols = cols; p.rms = rms; p.round_mode = round_mode;
+  p.mean_out = mean_out; p.rstd_out = rstd_out;
+  return ti::launch_rownorm<false>(p, (hipStream_t)stream);
+}
+
+int ti_dq_add_layernorm_q(const int32_t* acc, int64_t acc_row_stride, float in_scale, const float* resid_in,
+                          int64_t resid_in_row_stride, const float* gamma, const float* beta, float eps,
+                          float* resid_out, int64_t resid_out_row_stride, int8_t* y, int64_t y_row_stride,
+                          float* ln_out_f32, int64_t ln_out_row_stride, int rows, int cols, int round_mode,
+                          float* mean_out, float* rstd_out, void* stream) {
+  if (rows < 0 || cols < 0) return ti::fail(TI_E_SHAPE, "negative size");
+  if (rows == 0 || cols == 0) return TI_OK;
+  if (!acc || !resid_in || !resid_out || !gamma) return ti::fail(TI_E_NULL, "acc, resid_in, resid_out and gamma are required");
+  if (!y && !ln_out_f32) return ti::fail(TI_E_NULL, "one of y / ln_out_f32 is required");
+  if (round_mode != TI_ROUND_RNE_CLAMP && round_mode != TI_ROUND_TRUNC) return ti::fail(TI_E_COMBO, "round mode %d", round_mode);
+  ti::RowNormParams p = {};
+  p.acc = acc; p.acc_rs = acc_row_stride; p.in_scale = in_scale;
+  p.resid_in = resid_in; p.rin_rs = resid_in_row_stride;
+  p.resid_out = resid_out; p.rout_rs = resid_out_row_stride;
+  p.gamma = gamma; p.beta = beta; p.eps = eps;
+  p.y = y; p.y_rs = y_row_stride;
+  p.ln_out = ln_out_f32; p.ln_rs = ln_out_row_stride;
+  p.rows = rows; p.cols = cols; p.rms = 0; p.round_mode = round_mode;
+  p.mean_out = mean_out; p.rstd_out = rstd_out;
+  return ti::launch_rownorm<true>(p, (hipStream_t)stream);
+}
+
+int ti_gelu_q(const float* x, const float* scale, int8_t* y, int64_t n, int round_mode, void* stream) {
+  if (n < 0) return ti::fail(TI_E_SHAPE, "negative size");
+  if (n == 0) return TI_OK;
+  if (!x || !scale || !y) return ti::fail(TI_E_NULL, "x, scale and y are required");
+  if (round_mode != TI_ROUND_RNE_CLAMP && round_mode != TI_ROUND_TRUNC) return ti::fail(TI_E_COMBO, "round mode %d", round_mode);
+  int rc = ti::check_device();
+  if (rc != TI_OK) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  int64_t done = 0;
+  if ((((uintptr_t)x) & 15) == 0 && (((uintptr_t)y) & 3) == 0 && n >= 4) {
+    const int64_t nvec = n / 4;
+    int64_t blocks = (nvec + ti::GQ_THREADS * ti::GQ_UNROLL - 1) / (ti::GQ_THREADS * ti::GQ_UNROLL);
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    ti::gelu_q_vec_kernel<<<dim3((unsigned)blocks), dim3(ti::GQ_THREADS), 0, s>>>(x, scale, y, nvec, round_mode);
+    rc = ti::launch_status("gelu_q_vec_kernel");
+    if (rc != TI_OK) return rc;
+    done = nvec * 4;
+  }
+  if (done < n) {
+    int64_t blocks = (n - done + ti::GQ_THREADS - 1) / ti::GQ_THREADS;
+    if (blocks > 256 * 16) blocks = 256 * 16;
+    ti::gelu_q_any_kernel<<<dim3((unsigned)blocks), dim3(ti::GQ_THREADS), 0, s>>>(x, scale, y, done, n, round_mode);
+    rc = ti::launch_status("gelu_q_any_kernel");
+  }
+  return rc;
+}
+
+}  // extern "C"

@@ -1,0 +1,75 @@
+// ti_common.h — shared host/device helpers for libtriton_int_hip.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/triton_int_hip.h"
+
+namespace ti {
+
+// ---- host: error reporting ---------------------------------------------------------------
+void set_error(const char* fmt, ...);
+int fail(int code, const char* fmt, ...);
+// Checks once per device that the current device is gfx950; returns TI_OK or TI_E_DEVICE.
+int check_device();
+int launch_status(const char* what);
+
+// ---- device: quantisation helpers ----------------------------------------------------------
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+// clamp(round_half_even(v), -128, 127), NaN -> 0.  v_rndne_f32, v_cvt_i32_f32 (saturating,
+// NaN -> 0), v_med3_i32.  TRUNC drops the rndne: the conversion itself truncates toward zero.
+template <bool TRUNC>
+__device__ __forceinline__ int q8(float v) {
+  float r = TRUNC ? v : __builtin_rintf(v);
+  int i = (int)r;
+  return min(max(i, -128), 127);
+}
+
+__device__ __forceinline__ int q8(float v, int round_mode) {
+  return round_mode == TI_ROUND_TRUNC ? q8<true>(v) : q8<false>(v);
+}
+
+// fp32 -> int32 with the same two modes; the hardware conversion saturates and maps NaN to 0.
+__device__ __forceinline__ int q32(float v, int round_mode) {
+  float r = round_mode == TI_ROUND_TRUNC ? v : __builtin_rintf(v);
+  if (r >= 2147483648.0f) return 0x7fffffff;
+  if (r <= -2147483648.0f) return (int)0x80000000;
+  if (r != r) return 0;
+  return (int)r;
+}
+
+__device__ __forceinline__ unsigned pack4(int a, int b, int c, int d) {
+  return (unsigned)(a & 0xff) | ((unsigned)(b & 0xff) << 8) | ((unsigned)(c & 0xff) << 16) |
+         ((unsigned)d << 24);
+}
+
+// tanh-GELU times scale in the literal evaluation order of the reference
+// (kernels/fused.py:79): 0.5 * x * (1 + tanh(k * (x + 0.044715 * x * x * x))) * scale.
+__device__ __forceinline__ float gelu_tanh_scaled(float x, float scale) {
+  const float k = 0.79788456080286535588f;
+  float cube = ((0.044715f * x) * x) * x;
+  float inner = k * (x + cube);
+  float t = tanhf(inner);
+  return ((0.5f * x) * (1.0f + t)) * scale;
+}
+
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  unsigned u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
+  _Float16 h = (_Float16)f;  // v_cvt_f16_f32, round-to-nearest-even
+  return __builtin_bit_cast(uint16_t, h);
+}
+
+}  // namespace ti

@@ -1,0 +1,74 @@
+"""Shared launcher plumbing for the int8 GEMM / BMM entry point ti_bmm_i8."""
+from __future__ import annotations
+
+import torch
+
+from .. import _lib as L
+
+
+def launch_bmm(a3, b3, c3, *, epilogue, bias=None, alpha=None, beta=None, round_mode=L.ROUND_RNE_CLAMP,
+               config=-1):
+    """a3 [B,M,K] int8, b3 [B,N,K] int8 (logical; any strides), c3 [B,M,N] preallocated."""
+    L.require_cuda(a3, b3, c3, bias)
+    assert a3.dtype == torch.int8 and b3.dtype == torch.int8, "operands must be int8"
+    dev = a3.device
+    assert b3.device == dev and c3.device == dev, "operands must be on one device"
+    B, M, K = a3.shape
+    _, N, _ = b3.shape
+    bias_kind = L.BIAS_NONE
+    if bias is not None:
+        assert bias.device == dev
+        assert bias.numel() == N, "bias must have one element per output column"
+        bias = bias.contiguous()
+        bias_kind = L.TORCH_TO_BIAS[bias.dtype]
+    alpha_t = None if alpha is None else L.scale_tensor(alpha, dev)
+    beta_t = None if beta is None else L.scale_tensor(beta, dev)
+    with torch.cuda.device(dev):
+        rc = L.lib().ti_bmm_i8_config(
+            L.ptr(a3), a3.stride(0), a3.stride(1), a3.stride(2),
+            L.ptr(b3), b3.stride(0), b3.stride(1), b3.stride(2),
+            L.ptr(c3), c3.stride(0), c3.stride(1), c3.stride(2),
+            B, M, N, K, L.ptr(bias), bias_kind, L.ptr(alpha_t), L.ptr(beta_t),
+            int(epilogue), L.TORCH_TO_DT[c3.dtype], int(round_mode), int(config), L.current_stream(dev))
+    L.check(rc, "ti_bmm_i8")
+    return c3
+
+
+def linear(a, w, *, epilogue, out_dtype, bias=None, alpha=None, beta=None, out=None,
+           round_mode=L.ROUND_RNE_CLAMP, config=-1):
+    """Common body of the linear_* launchers (reference: kernels/linear.py:257-288 and siblings)."""
+    tmp_shape = a.shape[:-1]
+    assert len(w.shape) == 2
+    a = a.view(-1, a.shape[-1])
+    assert a.shape[1] == w.shape[1], "Incompatible dimensions"
+    M, K = a.shape
+    N, K = w.shape
+    if out is None:
+        c = torch.empty((M, N), device=a.device, dtype=out_dtype)
+    else:
+        assert out.dtype == out_dtype and out.numel() == M * N, "out has the wrong dtype or size"
+        c = out.view(M, N)
+    launch_bmm(a.unsqueeze(0), w.unsqueeze(0), c.unsqueeze(0), epilogue=epilogue, bias=bias, alpha=alpha,
+               beta=beta, round_mode=round_mode, config=config)
+    return c.view(*tmp_shape, N)
+
+
+def bmm(a, b, *, b_is_kn, epilogue, out_dtype, alpha=None, out=None, round_mode=L.ROUND_RNE_CLAMP, config=-1):
+    """Common body of the bmm_* launchers (reference: kernels/bmm.py:577-612 and siblings)."""
+    tmp_shape = a.shape[:-1]
+    assert len(a.shape) == 3 and len(b.shape) == 3
+    assert a.shape[0] == b.shape[0]
+    if b_is_kn:
+        assert a.shape[2] == b.shape[1], "Incompatible dimensions"
+        b = b.transpose(1, 2)  # logical [B,N,K] view of the [B,K,N] operand
+    else:
+        assert a.shape[2] == b.shape[2], "Incompatible dimensions"
+    _, M, K = a.shape
+    B, N, K = b.shape
+    if out is None:
+        c = torch.empty((B, M, N), device=a.device, dtype=out_dtype)
+    else:
+        assert out.dtype == out_dtype and out.shape == (B, M, N), "out has the wrong dtype or shape"
+        c = out
+    launch_bmm(a, b, c, epilogue=epilogue, alpha=alpha, round_mode=round_mode, config=config)
+    return c.view(*tmp_shape, N)

@@ -1,0 +1,105 @@
+"""Fused launchers — the int8 entries of triton_int/kernels/fused.py plus the two ops that file
+only sketches: the dequant + residual-add + LayerNorm + quantise kernel (its Triton stub at
+kernels/fused.py:17-61 is never launched) and a launchable stand-alone GELU-quant
+(fast_geluQ, kernels/fused.py:76-79, is a device function there).
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _lib as L
+from ._gemm import linear as _linear
+
+
+def linear_a8_w8_bfp32_ofp32_GeLu_Q(a, b, bias, scale_a, scale_b, out=None, *, _round_mode=L.ROUND_RNE_CLAMP,
+                                    _config=-1):
+    """x = scale_a * acc + bias_f32;  q8(gelu_tanh(x) * scale_b)   (reference: kernels/fused.py:197-231;
+    scale_b is 1/output_scale, nn/fused.py:148-150)."""
+    if bias is not None and bias.dtype != torch.float32:
+        bias = bias.to(torch.float32)
+    return _linear(a, b, epilogue=L.EPI_GELU_I8, out_dtype=torch.int8, bias=bias, alpha=scale_a, beta=scale_b,
+                   out=out, round_mode=_round_mode, config=_config)
+
+
+def layer_norm_fwd_fused_single_pass_q(x, weight, bias, eps, use_rms_norm=False, *, _round_mode=L.ROUND_RNE_CLAMP,
+                                       _return_stats=False):
+    """LayerNorm (or RMSNorm) over the last dim, output quantised to int8
+    (reference: kernels/fused.py:336-382)."""
+    assert x.dtype == weight.dtype, f"input and weight bias must have the same dtype: {x.dtype}, {weight.dtype}"
+    if bias is not None:
+        assert x.dtype == bias.dtype, f"input and bias must have the same dtype: {x.dtype}, {bias.dtype}"
+    assert x.dtype == torch.float32, "the int8 LayerNorm kernel takes fp32 activations (nn/fused.py:43)"
+    L.require_cuda(x, weight, bias)
+    N = x.shape[-1]
+    assert weight.numel() == N and (bias is None or bias.numel() == N)
+    a_arg = x.view(-1, N)
+    if a_arg.stride(1) != 1:
+        a_arg = a_arg.contiguous()
+    out = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    o2 = out.view(-1, N)
+    M = a_arg.shape[0]
+    weight = weight.contiguous()
+    bias = None if bias is None else bias.contiguous()
+    mean = rstd = None
+    if _return_stats:
+        mean = torch.empty(M, dtype=torch.float32, device=x.device)
+        rstd = torch.empty(M, dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = L.lib().ti_layernorm_q(L.ptr(a_arg), a_arg.stride(0) if M > 1 else N, L.ptr(weight), L.ptr(bias),
+                                    float(eps), L.ptr(o2), N, M, N, int(bool(use_rms_norm)), int(_round_mode),
+                                    L.ptr(mean), L.ptr(rstd), L.current_stream(x.device))
+    L.check(rc, "ti_layernorm_q")
+    return (out, mean, rstd) if _return_stats else out
+
+
+def dq_add_layernorm_q(input_int32, input_scale_fp, residual_input_fp, gamma, beta, eps, *, quantize=True,
+                       _round_mode=L.ROUND_RNE_CLAMP, _return_stats=False):
+    """residual_out = residual_in + input_scale * int32;  LayerNorm;  -> (residual_out fp32,
+    int8) — or the fp32 LayerNorm output when quantize=False.  Semantics of
+    functional/fused.py:6-24; the argument order is that of the intended native op,
+    functional/fused.py:27-32."""
+    L.require_cuda(input_int32, residual_input_fp, gamma, beta)
+    assert input_int32.dtype == torch.int32, "input_int32 must be int32"
+    assert input_int32.shape == residual_input_fp.shape, "Incompatible dimensions"
+    shape = input_int32.shape
+    H = shape[-1]
+    assert gamma.numel() == H and (beta is None or beta.numel() == H)
+    acc = input_int32.reshape(-1, H)
+    rin = residual_input_fp.to(torch.float32).reshape(-1, H)
+    if acc.stride(1) != 1:
+        acc = acc.contiguous()
+    if rin.stride(1) != 1:
+        rin = rin.contiguous()
+    rows = acc.shape[0]
+    dev = acc.device
+    gamma = gamma.to(torch.float32).contiguous()
+    beta = None if beta is None else beta.to(torch.float32).contiguous()
+    rout = torch.empty((rows, H), dtype=torch.float32, device=dev)
+    y = torch.empty((rows, H), dtype=torch.int8, device=dev) if quantize else None
+    ln = None if quantize else torch.empty((rows, H), dtype=torch.float32, device=dev)
+    mean = rstd = None
+    if _return_stats:
+        mean = torch.empty(rows, dtype=torch.float32, device=dev)
+        rstd = torch.empty(rows, dtype=torch.float32, device=dev)
+    if torch.is_tensor(input_scale_fp):
+        input_scale_fp = float(input_scale_fp)  # the module holds a python float (nn/fused.py:62)
+    with torch.cuda.device(dev):
+        rc = L.lib().ti_dq_add_layernorm_q(
+            L.ptr(acc), acc.stride(0) if rows > 1 else H, float(input_scale_fp), L.ptr(rin),
+            rin.stride(0) if rows > 1 else H, L.ptr(gamma), L.ptr(beta), float(eps), L.ptr(rout), H, L.ptr(y), H,
+            L.ptr(ln), H, rows, H, int(_round_mode), L.ptr(mean), L.ptr(rstd), L.current_stream(dev))
+    L.check(rc, "ti_dq_add_layernorm_q")
+    res = (rout.view(shape), (y if quantize else ln).view(shape))
+    return res + (mean, rstd) if _return_stats else res
+
+
+def gelu_q(x, scale, *, _round_mode=L.ROUND_RNE_CLAMP):
+    """q8(gelu_tanh(x) * scale) element-wise, x fp32 -> int8 (math of kernels/fused.py:76-79)."""
+    L.require_cuda(x)
+    x = x.to(torch.float32).contiguous()
+    y = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    s = L.scale_tensor(scale, x.device)
+    with torch.cuda.device(x.device):
+        rc = L.lib().ti_gelu_q(L.ptr(x), L.ptr(s), L.ptr(y), x.numel(), int(_round_mode), L.current_stream(x.device))
+    L.check(rc, "ti_gelu_q")
+    return y
