@@ -39,10 +39,12 @@ def linear(a, w, *, epilogue, out_dtype, bias=None, alpha=None, beta=None, out=N
     """Common body of the linear_* launchers (reference: kernels/linear.py:257-288 and siblings)."""
     tmp_shape = a.shape[:-1]
     assert len(w.shape) == 2
-    a = a.view(-1, a.shape[-1])
-    assert a.shape[1] == w.shape[1], "Incompatible dimensions"
-    M, K = a.shape
+    assert a.shape[-1] == w.shape[1], "Incompatible dimensions"
     N, K = w.shape
+    M = 1
+    for d in tmp_shape:
+        M *= d
+    a = a.view(M, K)
     if out is None:
         c = torch.empty((M, N), device=a.device, dtype=out_dtype)
     else:
