@@ -119,6 +119,9 @@ int ti_bmm_i8_config(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk,
                      int config, void* stream);
 int ti_gemm_num_configs(void);
 const char* ti_gemm_config_name(int config);
+/* Index of the configuration the calling thread's most recent ti_bmm_i8* launch used (-1 if
+ * none); lets a benchmark attribute time to the kernel that actually ran. */
+int ti_gemm_last_config(void);
 
 /* ---- row kernels ------------------------------------------------------------------- */
 

@@ -121,24 +121,28 @@ __device__ __forceinline__ EpiCtx make_epi(const GemmParams& p) {
 
 // ---- fast family -----------------------------------------------------------------------------
 //
-// LDS tile = ROWS x BK bytes, viewed as 16-byte chunks; chunk c of row r lives at chunk slot
-// c ^ ((r >> SWZ) & (CH-1)) of that row, which spreads the 16-byte reads of the 32 lanes that
-// share a chunk index (one MFMA operand column) over the banks.
+// LDS stage = A tile (BM x BK bytes) + B tile (BN x BK bytes), each viewed as 16-byte chunks;
+// chunk c of row r lives at chunk slot c ^ ((r >> SWZ) & (CH-1)) of that row, which spreads the
+// 16-byte reads of the 32 lanes that share a chunk index (one MFMA operand column) over the banks.
 //
-// Loads: chunk slot q = it*NT + tid of the tile is filled by thread tid.  LOADMODE 0 goes
-// through registers (buffer_load_dwordx4 + ds_write_b128); LOADMODE 1 lets the buffer load write
-// LDS itself (buffer_load_dwordx4 ... lds: lane i of a wave lands at M0-base + 16*i).
-// Buffer descriptors bound the loads: rows past M/N and the K tail read as zero.
+// Global -> LDS: chunk slot q = it*NT + tid of a tile is filled by thread tid with
+// buffer_load_dwordx4 ... lds (lane i of a wave lands at M0-base + 16*i, no VGPR round trip).
+// The buffer descriptors bound the loads: rows past M/N and the K tail read as zero.
+//
+// Pipeline: NSTAGE LDS stages, NSTAGE-1 k-tiles of loads in flight.  Per k-tile one barrier,
+// placed before the last MFMA k-step so that the first operand fragments of the next k-tile are
+// fetched from LDS while the matrix pipe is still busy; inside a k-tile the fragments of k-step
+// s+1 are read while the MFMAs of k-step s issue (two register sets).
 
 template <int ROWS, int BK, int NT, int SWZ>
 struct TileLoader {
   static constexpr int CH = BK / 16;
   static constexpr int IT = ROWS * CH / NT;
   static_assert(ROWS * CH % NT == 0, "tile must split evenly over the threads");
-  int voff[IT];  // byte offset of the chunk at k-tile 0; advanced by BK per k-tile
-  int kpos[IT];  // k index of the chunk at k-tile 0
+  int voff[IT];  // byte offset of this thread's chunk in k-tile 0 (the k offset is added as a scalar)
+  int klim[IT];  // the chunk is inside K while k0 < klim
 
-  __device__ __forceinline__ void init(int tid, int row0, int ld) {
+  __device__ __forceinline__ void init(int tid, int row0, int ld, int K) {
 #pragma unroll
     for (int it = 0; it < IT; ++it) {
       const int q = it * NT + tid;
@@ -146,12 +150,42 @@ struct TileLoader {
       const int cphys = q % CH;
       const int clog = cphys ^ ((row >> SWZ) & (CH - 1));
       voff[it] = (row0 + row) * ld + clog * 16;
-      kpos[it] = clog * 16;
+      klim[it] = K - clog * 16;
     }
   }
 };
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int SWZ, int LOADMODE, int OUTCLS>
+// The global -> LDS loads and the waits on them are written as inline assembly on purpose.  For
+// the builtin form the compiler tracks "LDS written by a buffer load" conservatively: every
+// workgroup barrier, and every LDS read that might alias, gets an s_waitcnt vmcnt(0) in front of
+// it, which drains the load pipeline once per k-tile and defeats multi-stage prefetching.  With
+// the loads invisible to that tracking, the kernel counts them itself (vmcnt retires in order).
+// M0 carries the LDS destination of a wave's 64 x 16 bytes; nothing else in these kernels uses M0.
+__device__ __forceinline__ v4i make_rsrc(const void* base, int bytes) {
+  const uint64_t a = (uint64_t)base;
+  v4i r;
+  r[0] = (int)(uint32_t)a;
+  r[1] = (int)((uint32_t)(a >> 32) & 0xffffu);  // stride 0: raw buffer
+  r[2] = bytes;                                 // num_records: loads at or past it return 0
+  r[3] = 0x00020000;                            // 32-bit data format word of gfx9-family raw buffers
+  return r;
+}
+
+__device__ __forceinline__ void dma16_to_lds(v4i rsrc, int voff, int soff, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+               : "memory");
+}
+
+// wait until at most N of this wave's buffer loads are outstanding and its LDS reads are done,
+// then meet the other waves of the workgroup
+template <int N>
+__device__ __forceinline__ void wait_loads_and_barrier() {
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int SWZ, int NSTAGE, int OUTCLS>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmParams p) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int CH = BK / 16;
@@ -161,8 +195,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmPa
   constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
   constexpr int STAGE = A_BYTES + B_BYTES;
   constexpr int C_PITCH = BN + 4;  // int8 staging pitch: 33-dword rows keep dword writes conflict-free
-  constexpr int LDS_BYTES = (2 * STAGE > BM * C_PITCH) ? 2 * STAGE : BM * C_PITCH;
-  static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % 32 == 0, "tile shape");
+  constexpr int LDS_BYTES = (NSTAGE * STAGE > BM * C_PITCH) ? NSTAGE * STAGE : BM * C_PITCH;
+  constexpr int DEPTH = NSTAGE - 1;  // k-tiles of loads in flight
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % 64 == 0, "tile shape");
+  static_assert(NSTAGE >= 3 && LDS_BYTES <= 160 * 1024, "LDS budget");
 
   __shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];
 
@@ -182,55 +218,41 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmPa
   // bytes addressable from the batch base: rows past the end and the K tail read as zero
   const int a_extent = (p.M - 1) * lda + p.K;
   const int b_extent = (p.N - 1) * ldb + p.K;
-  __amdgpu_buffer_rsrc_t rA = __builtin_amdgcn_make_buffer_rsrc((void*)Ab, 0, a_extent, 0x00020000);
-  __amdgpu_buffer_rsrc_t rB = __builtin_amdgcn_make_buffer_rsrc((void*)Bb, 0, b_extent, 0x00020000);
+  const v4i rA = make_rsrc(Ab, a_extent);
+  const v4i rB = make_rsrc(Bb, b_extent);
+  const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+  // LDS byte address of this wave's 1 KB slot in chunk-slot group 0 of stage 0
+  const unsigned wave_slot = __builtin_amdgcn_readfirstlane(lds_base + wave * 1024);
 
   TileLoader<BM, BK, NT, SWZ> la;
   TileLoader<BN, BK, NT, SWZ> lb;
-  la.init(tid, m0, lda);
-  lb.init(tid, n0, ldb);
+  la.init(tid, m0, lda, p.K);
+  lb.init(tid, n0, ldb, p.K);
   constexpr int A_IT = decltype(la)::IT, B_IT = decltype(lb)::IT;
+  constexpr int LOADS = A_IT + B_IT;  // buffer loads per thread per k-tile
   const int KT = (p.K + BK - 1) / BK;
   const int OOB = (int)0x80000000;
 
-  v4u ra[LOADMODE == 0 ? A_IT : 1], rb[LOADMODE == 0 ? B_IT : 1];
-
-  // issue the loads of k-tile kt (into registers, or straight into LDS stage `st`)
-  auto issue = [&](int kt, int st) {
-    const int k0 = kt * BK;
-    char* sA = lds + st * STAGE;
-    char* sB = sA + A_BYTES;
-#pragma unroll
-    for (int it = 0; it < A_IT; ++it) {
-      const int vo = (k0 + la.kpos[it] < p.K) ? la.voff[it] + k0 : OOB;
-      if constexpr (LOADMODE == 0) {
-        ra[it] = __builtin_amdgcn_raw_buffer_load_b128(rA, vo, 0, 0);
-      } else {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(
-            rA, (void __attribute__((address_space(3)))*)(sA + (it * NT + wave * 64) * 16), 16, vo, 0, 0, 0);
-      }
-    }
-#pragma unroll
-    for (int it = 0; it < B_IT; ++it) {
-      const int vo = (k0 + lb.kpos[it] < p.K) ? lb.voff[it] + k0 : OOB;
-      if constexpr (LOADMODE == 0) {
-        rb[it] = __builtin_amdgcn_raw_buffer_load_b128(rB, vo, 0, 0);
-      } else {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(
-            rB, (void __attribute__((address_space(3)))*)(sB + (it * NT + wave * 64) * 16), 16, vo, 0, 0, 0);
-      }
+  // One global -> LDS load of the k-tile being fetched (k offset k_issue, LDS stage st_issue):
+  // load number d of the LOADS this thread owns per k-tile.  The address is the thread's constant
+  // byte offset plus the scalar k offset; a chunk at or past K is redirected out of bounds so it
+  // reads as zero instead of running into the next row.  Past the end of K every chunk is out of bounds:
+  // the loads write zeros into a stage nobody reads again, which keeps the number of loads in
+  // flight, and so the vmcnt to wait for, constant.
+  int k_issue = 0, st_issue = 0;
+  auto dma = [&](int d) {
+    if (d < A_IT) {
+      const unsigned dst = wave_slot + st_issue * STAGE + d * NT * 16;
+      dma16_to_lds(rA, (k_issue < la.klim[d]) ? la.voff[d] : OOB, k_issue, dst);
+    } else {
+      const int e = d - A_IT;
+      const unsigned dst = wave_slot + st_issue * STAGE + A_BYTES + e * NT * 16;
+      dma16_to_lds(rB, (k_issue < lb.klim[e]) ? lb.voff[e] : OOB, k_issue, dst);
     }
   };
-  // LOADMODE 0 only: registers -> LDS stage st
-  auto commit = [&](int st) {
-    if constexpr (LOADMODE == 0) {
-      char* sA = lds + st * STAGE;
-      char* sB = sA + A_BYTES;
-#pragma unroll
-      for (int it = 0; it < A_IT; ++it) *(v4u*)(sA + (it * NT + tid) * 16) = ra[it];
-#pragma unroll
-      for (int it = 0; it < B_IT; ++it) *(v4u*)(sB + (it * NT + tid) * 16) = rb[it];
-    }
+  auto dma_advance = [&]() {
+    k_issue += BK;
+    st_issue = (st_issue + 1 == NSTAGE) ? 0 : st_issue + 1;
   };
 
   v16i acc[TM][TN];
@@ -247,44 +269,85 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmPa
   const int fsw = (frow >> SWZ) & (CH - 1);
   const int fhalf = lane >> 5;
   const int a_lane = (wm * WTM + frow) * BK;
-  const int b_lane = (wn * WTN + frow) * BK;
+  const int b_lane = A_BYTES + (wn * WTN + frow) * BK;
+
+  v4i fa[2][TM], fb[2][TN];
+  // fragment number r (A blocks first, then B blocks) of k-step ks of the stage -> register set buf
+  auto load_frag = [&](const char* stage, int ks, int buf, int r) {
+    const int coff = ((ks * 2 + fhalf) ^ fsw) * 16;
+    if (r < TM) fa[buf][r] = *(const v4i*)(stage + a_lane + r * 32 * BK + coff);
+    else fb[buf][r - TM] = *(const v4i*)(stage + b_lane + (r - TM) * 32 * BK + coff);
+  };
+  auto mfma = [&](int buf, int u) {
+    const int i = u / TN, j = u % TN;
+    if constexpr (OUTCLS == OUT8)  // rows of the MFMA result = n (4 consecutive n per lane)
+      acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
+    else  // rows of the MFMA result = m, lanes run along n
+      acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
+  };
+  constexpr int NM = TM * TN, NR = TM + TN;
+  // One k-step, pinned instruction order: MFMA u, then fragment read u for the next k-step, and
+  // ND global->LDS loads spread evenly between the MFMAs.  A wave can only push one such load
+  // into the memory pipeline every ~64 cycles, so loads issued back to back stall the wave's
+  // instruction stream (and with it the matrix pipe); two or three MFMAs between loads hide it.
+  auto kstep = [&](int buf, const char* rd_stage, int rd_ks, bool do_read, int d0, int nd) {
+    int d = 0;
+#pragma unroll
+    for (int u = 0; u < NM; ++u) {
+      mfma(buf, u);
+      if (do_read) {
+#pragma unroll
+        for (int r = 0; r < NR; ++r)
+          if (r * NM / NR == u || (NM > NR && r == u)) {
+            if (NM > NR ? r == u : r * NM / NR == u) load_frag(rd_stage, rd_ks, buf ^ 1, r);
+          }
+      }
+      if (d < nd && (u + 1) * nd >= (d + 1) * NM) {
+        dma(d0 + d);
+        ++d;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // loads of one k-tile are split over the k-steps: the last k-step (after the barrier) gets
+  // LOADS_B of them, the others LOADS_A in total
+  constexpr int PER_KS = (LOADS + KS - 1) / KS;
+  constexpr int LOADS_B = (LOADS - PER_KS * (KS - 1) > 0) ? LOADS - PER_KS * (KS - 1) : 0;
+  constexpr int LOADS_A = LOADS - LOADS_B;
 
   if (KT > 0) {
-    issue(0, 0);
-    if constexpr (LOADMODE == 0) commit(0);
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < DEPTH; ++t) {
+#pragma unroll
+      for (int d = 0; d < LOADS; ++d) dma(d);
+      dma_advance();
+    }
+    wait_loads_and_barrier<LOADS*(DEPTH - 1)>();
+#pragma unroll
+    for (int r = 0; r < NR; ++r) load_frag(lds, 0, 0, r);
   }
 
+  int st = 0;
   for (int kt = 0; kt < KT; ++kt) {
-    const int st = kt & 1;
-    if (kt + 1 < KT) issue(kt + 1, st ^ 1);
-    const char* sA = lds + st * STAGE;
-    const char* sB = sA + A_BYTES;
+    const char* cur = lds + st * STAGE;
+    st = (st + 1 == NSTAGE) ? 0 : st + 1;
+    // k-steps 0 .. KS-2: read the fragments of the following k-step, fetch part A of k-tile kt+DEPTH
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const int coff = ((ks * 2 + fhalf) ^ fsw) * 16;
-      v4i fa[TM], fb[TN];
-#pragma unroll
-      for (int i = 0; i < TM; ++i) fa[i] = *(const v4i*)(sA + a_lane + i * 32 * BK + coff);
-#pragma unroll
-      for (int j = 0; j < TN; ++j) fb[j] = *(const v4i*)(sB + b_lane + j * 32 * BK + coff);
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-          if constexpr (OUTCLS == OUT8)  // rows of the MFMA result = n (4 consecutive n per lane)
-            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[j], fa[i], acc[i][j], 0, 0, 0);
-          else  // rows of the MFMA result = m, lanes run along n
-            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
-        }
+    for (int ks = 0; ks < KS - 1; ++ks) {
+      const int d0 = ks * PER_KS;
+      const int nd = (d0 + PER_KS <= LOADS_A) ? PER_KS : (LOADS_A - d0 > 0 ? LOADS_A - d0 : 0);
+      kstep(ks & 1, cur, ks + 1, true, d0, nd);
     }
-    if (kt + 1 < KT) {
-      if constexpr (LOADMODE == 0) commit(st ^ 1);
-      else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
-    __syncthreads();
+    // every LDS read of this k-tile is issued.  Wait for them and for k-tile kt+1 to have landed
+    // (younger loads may stay in flight), then let the workgroup agree: after the barrier the
+    // stage of k-tile kt+1 is readable and this k-tile's stage may be overwritten.
+    wait_loads_and_barrier<LOADS*(DEPTH - 2) + LOADS_A>();
+    // last k-step: first fragments of the next k-tile, part B of the fetch
+    kstep((KS - 1) & 1, lds + st * STAGE, 0, kt + 1 < KT, LOADS_A, LOADS_B);
+    dma_advance();
   }
+  // the trailing (out-of-bounds) loads still write zeros into LDS: drain before re-using it
+  wait_loads_and_barrier<0>();
 
   // ---- epilogue ----
   const EpiCtx e = make_epi(p);
@@ -431,27 +494,26 @@ struct Config {
   bool fast;       // needs the aligned K-contiguous layout
 };
 
-#define TI_FAST(BM, BN, BK, WM, WN, SWZ, LM)                                              \
+#define TI_FAST(BM, BN, BK, WM, WN, SWZ, NS)                                              \
   {                                                                                       \
-    "mfma_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN "_s" #SWZ "_l" #LM,                        \
-        {gemm_mfma_kernel<BM, BN, BK, WM, WN, SWZ, LM, OUT8>,                               \
-         gemm_mfma_kernel<BM, BN, BK, WM, WN, SWZ, LM, OUT32>,                              \
-         gemm_mfma_kernel<BM, BN, BK, WM, WN, SWZ, LM, OUT16>},                             \
+    "mfma_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN "_s" #SWZ "_p" #NS,                        \
+        {gemm_mfma_kernel<BM, BN, BK, WM, WN, SWZ, NS, OUT8>,                               \
+         gemm_mfma_kernel<BM, BN, BK, WM, WN, SWZ, NS, OUT32>,                              \
+         gemm_mfma_kernel<BM, BN, BK, WM, WN, SWZ, NS, OUT16>},                             \
         BM, BN, BK, WM * WN * 64, true                                                    \
   }
 
 static const Config g_configs[] = {
     {"gather_64x64x32", {gemm_gather_kernel<OUT8>, gemm_gather_kernel<OUT32>, gemm_gather_kernel<OUT16>}, 64, 64, 32, 256, false},
-    TI_FAST(256, 128, 128, 2, 2, 0, 0),
-    TI_FAST(256, 128, 128, 2, 2, 0, 1),
-    TI_FAST(256, 128, 128, 2, 2, 1, 1),
-    TI_FAST(128, 128, 128, 2, 2, 0, 0),
-    TI_FAST(128, 128, 128, 2, 2, 0, 1),
-    TI_FAST(256, 128, 64, 2, 2, 1, 0),
-    TI_FAST(256, 128, 64, 2, 2, 1, 1),
-    TI_FAST(256, 128, 64, 2, 2, 2, 1),
-    TI_FAST(128, 256, 128, 2, 2, 0, 1),
-    TI_FAST(64, 64, 128, 2, 2, 0, 1),
+    TI_FAST(256, 128, 128, 2, 2, 1, 3),
+    TI_FAST(256, 128, 128, 2, 2, 0, 3),
+    TI_FAST(256, 128, 64, 2, 2, 2, 4),
+    TI_FAST(256, 128, 64, 2, 2, 2, 3),
+    TI_FAST(128, 128, 128, 2, 2, 1, 3),
+    TI_FAST(128, 128, 64, 2, 2, 2, 4),
+    TI_FAST(128, 256, 128, 2, 2, 1, 3),
+    TI_FAST(256, 256, 64, 2, 2, 2, 3),
+    TI_FAST(64, 64, 128, 2, 2, 1, 3),
 };
 static const int g_num_configs = (int)(sizeof(g_configs) / sizeof(g_configs[0]));
 
@@ -483,13 +545,13 @@ static int pick_config(const GemmParams& p) {
   // Largest tile that still gives every CU work; measured preferences are encoded as the
   // candidate order.
   const int64_t cus = 256;
-  const int cand[] = {2, 5, 10};
+  const int cand[] = {1, 5, 9};
   for (int c : cand) {
     const Config& k = g_configs[c];
     const int64_t tiles = (int64_t)((p.M + k.bm - 1) / k.bm) * ((p.N + k.bn - 1) / k.bn) * p.batch;
-    if (tiles >= cus || c == 10) return c;
+    if (tiles >= cus || c == 9) return c;
   }
-  return 10;
+  return 9;
 }
 
 static int pick_group_m(const GemmParams& p, const Config& k) {
@@ -536,6 +598,8 @@ static int validate(const GemmParams& p) {
   return TI_OK;
 }
 
+static thread_local int g_last_config = -1;
+
 static int run(GemmParams p, int config, hipStream_t stream) {
   int rc = validate(p);
   if (rc != TI_OK) return rc;
@@ -552,6 +616,7 @@ static int run(GemmParams p, int config, hipStream_t stream) {
   if ((int64_t)p.tiles_m * p.tiles_n > 0x7fffffff) return fail(TI_E_SHAPE, "too many tiles");
   p.group_m = pick_group_m(p, k);
   dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)p.batch, 1);
+  g_last_config = config;
   k.fn[out_class(p.out_dtype)]<<<grid, dim3(k.threads), 0, stream>>>(p);
   return launch_status(k.name);
 }
@@ -586,6 +651,8 @@ int ti_bmm_i8(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk, const int8
 }
 
 int ti_gemm_num_configs(void) { return ti::g_num_configs; }
+
+int ti_gemm_last_config(void) { return ti::g_last_config; }
 
 const char* ti_gemm_config_name(int config) {
   return (config >= 0 && config < ti::g_num_configs) ? ti::g_configs[config].name : "";
