@@ -11,6 +11,8 @@
 //
 // C = epilogue(sum_k A[m,k] * B[n,k]); A is [M,K], B is [N,K] (the reference's "N" operand,
 // kernels/linear.py:217), the "T" operand [K,N] arrives as strides (sBn = 1, sBk = N).
+#include <type_traits>
+
 #include "ti_common.h"
 
 namespace ti {
@@ -30,6 +32,11 @@ struct GemmParams {
 };
 
 enum OutClass { OUT8 = 0, OUT32 = 1, OUT16 = 2 };
+
+#ifdef TI_TRACE
+// debug builds only: per-wave cycle counts of the main loop (never compiled into the product)
+__device__ unsigned long long ti_trace_buf[8192];
+#endif
 
 // ---- tile -> (m, n) mapping ----------------------------------------------------------------
 // Workgroups are dealt round-robin to the 8 XCDs (each with a private L2), so consecutive
@@ -57,23 +64,34 @@ struct EpiCtx {
   float alpha, beta;
   int epilogue, round_mode, bias_kind;
   const void* bias;
+  const float* safe;  // always-readable 4 bytes (the A operand), target of the no-bias dummy loads
 };
 
-__device__ __forceinline__ float load_bias_f(const EpiCtx& e, int n) {
-  switch (e.bias_kind) {
-    case TI_BIAS_I8: return (float)((const int8_t*)e.bias)[n];
-    case TI_BIAS_I32: return (float)((const int32_t*)e.bias)[n];
-    case TI_BIAS_F32: return ((const float*)e.bias)[n];
-    default: return 0.0f;
-  }
+// Per-column term that is added to alpha*f(acc): beta*f(bias) for the scale epilogues, the raw
+// fp32 bias for GELU-Q (kernels/fused.py:184-186 adds the bias un-scaled), 0 without a bias.
+// KIND is the bias element type the caller has already branched on; without a bias the load is
+// redirected to element 0 of a valid buffer and the result replaced by 0, so there is no branch.
+template <int KIND>
+__device__ __forceinline__ float column_term_t(const EpiCtx& e, int n, bool gelu) {
+  const bool has = e.bias_kind != TI_BIAS_NONE;
+  const void* base = has ? e.bias : (const void*)e.safe;
+  const int idx = has ? n : 0;
+  float b;
+  if constexpr (KIND == TI_BIAS_I8) b = (float)((const int8_t*)base)[idx];
+  else if constexpr (KIND == TI_BIAS_I32) b = (float)((const int32_t*)base)[idx];
+  else b = ((const float*)base)[idx];
+  const float scaled = gelu ? b : b * e.beta;
+  return has ? scaled : 0.0f;
 }
 
-// Per-column term that is added to alpha*f(acc): beta*f(bias) for the scale epilogues, the raw
-// fp32 bias for GELU-Q (kernels/fused.py:184-186 adds the bias un-scaled).
 __device__ __forceinline__ float column_term(const EpiCtx& e, int n) {
-  if (e.bias_kind == TI_BIAS_NONE) return 0.0f;
-  float b = load_bias_f(e, n);
-  return e.epilogue == TI_EPI_GELU_I8 ? b : b * e.beta;
+  const bool gelu = e.epilogue == TI_EPI_GELU_I8;
+  switch (e.bias_kind) {
+    case TI_BIAS_I8: return column_term_t<TI_BIAS_I8>(e, n, gelu);
+    case TI_BIAS_I32: return column_term_t<TI_BIAS_I32>(e, n, gelu);
+    case TI_BIAS_F32: return column_term_t<TI_BIAS_F32>(e, n, gelu);
+    default: return 0.0f;
+  }
 }
 
 __device__ __forceinline__ float epi_value(const EpiCtx& e, int acc, float col) {
@@ -116,6 +134,7 @@ __device__ __forceinline__ EpiCtx make_epi(const GemmParams& p) {
   e.round_mode = p.round_mode;
   e.bias_kind = p.bias ? p.bias_kind : TI_BIAS_NONE;
   e.bias = p.bias;
+  e.safe = (const float*)p.A;
   return e;
 }
 
@@ -201,6 +220,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmPa
   static_assert(NSTAGE >= 3 && LDS_BYTES <= 160 * 1024, "LDS budget");
 
   __shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];
+#ifdef TI_TRACE
+  const uint64_t tr_entry = wall_clock64();
+#endif
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -241,6 +263,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmPa
   // flight, and so the vmcnt to wait for, constant.
   int k_issue = 0, st_issue = 0;
   auto dma = [&](int d) {
+#if defined(TI_ABLATE) && TI_ABLATE == 1
+    return;  // debug build: no global loads
+#endif
     if (d < A_IT) {
       const unsigned dst = wave_slot + st_issue * STAGE + d * NT * 16;
       dma16_to_lds(rA, (k_issue < la.klim[d]) ? la.voff[d] : OOB, k_issue, dst);
@@ -280,6 +305,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmPa
   };
   auto mfma = [&](int buf, int u) {
     const int i = u / TN, j = u % TN;
+#if defined(TI_ABLATE) && TI_ABLATE == 2
+    acc[i][j][0] += fa[buf][i][0] ^ fb[buf][j][0];  // debug build: no MFMA, keep the operands live
+    return;
+#endif
     if constexpr (OUTCLS == OUT8)  // rows of the MFMA result = n (4 consecutive n per lane)
       acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
     else  // rows of the MFMA result = m, lanes run along n
@@ -327,6 +356,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmPa
     for (int r = 0; r < NR; ++r) load_frag(lds, 0, 0, r);
   }
 
+#ifdef TI_TRACE
+  uint64_t tr_wait = 0, tr_bar = 0, tr_t0 = __builtin_readcyclecounter(), tr_w0 = wall_clock64();
+#endif
   int st = 0;
   for (int kt = 0; kt < KT; ++kt) {
     const char* cur = lds + st * STAGE;
@@ -341,40 +373,79 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmPa
     // every LDS read of this k-tile is issued.  Wait for them and for k-tile kt+1 to have landed
     // (younger loads may stay in flight), then let the workgroup agree: after the barrier the
     // stage of k-tile kt+1 is readable and this k-tile's stage may be overwritten.
+#ifdef TI_TRACE
+    const uint64_t tr_a = __builtin_readcyclecounter();
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LOADS*(DEPTH - 2) + LOADS_A) : "memory");
+    const uint64_t tr_b = __builtin_readcyclecounter();
+    asm volatile("s_barrier" ::: "memory");
+    const uint64_t tr_c = __builtin_readcyclecounter();
+    tr_wait += tr_b - tr_a;
+    tr_bar += tr_c - tr_b;
+#else
     wait_loads_and_barrier<LOADS*(DEPTH - 2) + LOADS_A>();
+#endif
     // last k-step: first fragments of the next k-tile, part B of the fetch
     kstep((KS - 1) & 1, lds + st * STAGE, 0, kt + 1 < KT, LOADS_A, LOADS_B);
     dma_advance();
   }
+#ifdef TI_TRACE
+  const uint64_t tr_t1 = __builtin_readcyclecounter(), tr_w1 = wall_clock64();
+#endif
   // the trailing (out-of-bounds) loads still write zeros into LDS: drain before re-using it
   wait_loads_and_barrier<0>();
 
   // ---- epilogue ----
+#ifdef TI_TRACE
+  if (lane == 0 && blockIdx.x < 256) {
+    unsigned long long* t = ti_trace_buf + (blockIdx.x * 4 + wave) * 8;
+    t[0] = tr_t1 - tr_t0; t[1] = tr_wait; t[2] = tr_bar; t[3] = tr_entry; t[4] = tr_w0; t[5] = tr_w1 - tr_w0;
+  }
+#endif
+  // The per-element code below is fully unrolled over the accumulator registers, so everything
+  // that depends on the epilogue kind is decided once, outside the unrolled part: one uniform
+  // branch selects a specialised body, and the remaining run-time options (rounding mode, ReLU,
+  // bias present) are folded into branch-free selects.
   const EpiCtx e = make_epi(p);
   char* Cb = (char*)p.C;
   const int lrow = lane & 31, lhi = lane >> 5;
+  const bool trunc = e.round_mode == TI_ROUND_TRUNC;
+  const bool has_bias = e.bias_kind != TI_BIAS_NONE;
 
   if constexpr (OUTCLS == OUT8) {
     // acc[i][j][r]: m = m0 + wm*WTM + i*32 + lrow;  n = n0 + wn*WTN + j*32 + 8*(r/4) + 4*lhi + r%4.
     // Quantise, pack 4 consecutive n into a dword, stage the tile in LDS, then write rows with
     // 16-byte stores.  (The K loop ended with a barrier, so the operand stages are free.)
+    const int q_floor = e.epilogue == TI_EPI_SCALE_RELU_I8 ? 0 : -128;  // ReLU = clamp from below at 0
+    auto body = [&](auto gelu_tag) {
+      constexpr bool GELU = decltype(gelu_tag)::value;
+      auto one = [&](int a, float col) -> int {
+        float v = (float)a * e.alpha;
+        v = col + v;  // col is 0 without a bias; adding it cannot change the quantised value
+        if constexpr (GELU) v = gelu_tanh_scaled(v, e.beta);
+        const float r = trunc ? v : __builtin_rintf(v);
+        return min(max((int)r, q_floor), 127);
+      };
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
+      for (int j = 0; j < TN; ++j) {
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int nl = wn * WTN + j * 32 + 8 * g + 4 * lhi;
-        float col[4];
+        for (int g = 0; g < 4; ++g) {
+          const int nl = wn * WTN + j * 32 + 8 * g + 4 * lhi;
+          float col[4];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) col[t] = column_term(e, min(n0 + nl + t, p.N - 1));
+          for (int t = 0; t < 4; ++t)
+            col[t] = column_term_t<GELU ? TI_BIAS_F32 : TI_BIAS_I8>(e, min(n0 + nl + t, p.N - 1), GELU);
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
-          const int ml = wm * WTM + i * 32 + lrow;
-          const unsigned w = pack4(epi_q8(e, acc[i][j][4 * g + 0], col[0]), epi_q8(e, acc[i][j][4 * g + 1], col[1]),
-                                   epi_q8(e, acc[i][j][4 * g + 2], col[2]), epi_q8(e, acc[i][j][4 * g + 3], col[3]));
-          *(unsigned*)(lds + ml * C_PITCH + nl) = w;
+          for (int i = 0; i < TM; ++i) {
+            const int ml = wm * WTM + i * 32 + lrow;
+            const unsigned w = pack4(one(acc[i][j][4 * g + 0], col[0]), one(acc[i][j][4 * g + 1], col[1]),
+                                     one(acc[i][j][4 * g + 2], col[2]), one(acc[i][j][4 * g + 3], col[3]));
+            *(unsigned*)(lds + ml * C_PITCH + nl) = w;
+          }
         }
       }
-    }
+    };
+    if (e.epilogue == TI_EPI_GELU_I8) body(std::true_type{});
+    else body(std::false_type{});
     __syncthreads();
     int8_t* Cz = (int8_t*)Cb + (int64_t)bz * p.sCb;
     const bool vec_ok = ((p.sCm & 15) == 0) && ((((uintptr_t)Cz) & 15) == 0);
@@ -398,23 +469,51 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmPa
     // acc[i][j][r]: m = m0 + wm*WTM + i*32 + 8*(r/4) + 4*lhi + r%4;  n = n0 + wn*WTN + j*32 + lrow.
     constexpr int ESZ = OUTCLS == OUT32 ? 4 : 2;
     char* Cz = Cb + (int64_t)bz * p.sCb * ESZ;
+    // KIND: 0 raw int32 (+ int32 bias), 1 scaled -> int32, 2 scaled -> fp32, 3 -> fp16, 4 -> bf16
+    auto body = [&](auto kind_tag) {
+      constexpr int KIND = decltype(kind_tag)::value;
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int n = n0 + wn * WTN + j * 32 + lrow;
-      const int nc = min(n, p.N - 1);
-      const float col = column_term(e, nc);
-      const int bias_i32 = (e.epilogue == TI_EPI_I32 && e.bias_kind == TI_BIAS_I32) ? ((const int*)e.bias)[nc] : 0;
+      for (int j = 0; j < TN; ++j) {
+        const int n = n0 + wn * WTN + j * 32 + lrow;
+        const int nc = min(n, p.N - 1);
+        const float col = KIND == 0 ? 0.0f : column_term_t<KIND == 1 ? TI_BIAS_I32 : TI_BIAS_F32>(e, nc, false);
+        const int bias_i32 = (KIND == 0 && e.bias_kind == TI_BIAS_I32) ? ((const int*)e.bias)[nc] : 0;
+        const bool n_ok = n < p.N;
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
+        for (int i = 0; i < TM; ++i) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int m = m0 + wm * WTM + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
-          if (m < p.M && n < p.N)
-            store_one<OUTCLS>(e, Cz, (int64_t)m * p.sCm + (int64_t)n * p.sCn, acc[i][j][r], col, bias_i32, p.out_dtype);
+          for (int r = 0; r < 16; ++r) {
+            const int m = m0 + wm * WTM + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+            if (!(n_ok && m < p.M)) continue;
+            const int64_t off = (int64_t)m * p.sCm + (int64_t)n * p.sCn;
+            const int a = acc[i][j][r];
+            if constexpr (KIND == 0) {
+              ((int*)Cz)[off] = (int)((unsigned)a + (unsigned)bias_i32);
+            } else {
+              float v = (float)a * e.alpha;
+              const float vb = col + v;
+              v = has_bias ? vb : v;
+              if constexpr (KIND == 1) ((int*)Cz)[off] = q32(v, e.round_mode);
+              else if constexpr (KIND == 2) ((float*)Cz)[off] = v;
+              else if constexpr (KIND == 3) ((uint16_t*)Cz)[off] = f32_to_f16_bits(v);
+              else ((uint16_t*)Cz)[off] = f32_to_bf16_bits(v);
+            }
+          }
         }
       }
+    };
+    if constexpr (OUTCLS == OUT32) {
+      if (e.epilogue == TI_EPI_I32) body(std::integral_constant<int, 0>{});
+      else if (e.epilogue == TI_EPI_SCALE_I32) body(std::integral_constant<int, 1>{});
+      else body(std::integral_constant<int, 2>{});
+    } else {
+      if (p.out_dtype == TI_F16) body(std::integral_constant<int, 3>{});
+      else body(std::integral_constant<int, 4>{});
     }
   }
+#ifdef TI_TRACE
+  if (lane == 0 && blockIdx.x < 256) ti_trace_buf[(blockIdx.x * 4 + wave) * 8 + 6] = wall_clock64();
+#endif
 }
 
 // ---- gather family -----------------------------------------------------------------------------
@@ -505,15 +604,14 @@ struct Config {
 
 static const Config g_configs[] = {
     {"gather_64x64x32", {gemm_gather_kernel<OUT8>, gemm_gather_kernel<OUT32>, gemm_gather_kernel<OUT16>}, 64, 64, 32, 256, false},
-    TI_FAST(256, 128, 128, 2, 2, 1, 3),
-    TI_FAST(256, 128, 128, 2, 2, 0, 3),
-    TI_FAST(256, 128, 64, 2, 2, 2, 4),
-    TI_FAST(256, 128, 64, 2, 2, 2, 3),
-    TI_FAST(128, 128, 128, 2, 2, 1, 3),
-    TI_FAST(128, 128, 64, 2, 2, 2, 4),
-    TI_FAST(128, 256, 128, 2, 2, 1, 3),
-    TI_FAST(256, 256, 64, 2, 2, 2, 3),
-    TI_FAST(64, 64, 128, 2, 2, 1, 3),
+    TI_FAST(256, 128, 128, 2, 2, 1, 3),  // 1
+    TI_FAST(256, 128, 128, 4, 2, 1, 3),  // 2
+    TI_FAST(256, 128, 128, 2, 4, 1, 3),  // 3
+    TI_FAST(256, 256, 64, 2, 4, 2, 3),   // 4
+    TI_FAST(256, 256, 64, 4, 2, 2, 3),   // 5
+    TI_FAST(128, 128, 64, 2, 2, 2, 4),   // 6
+    TI_FAST(128, 128, 128, 2, 2, 1, 3),  // 7
+    TI_FAST(64, 64, 128, 2, 2, 1, 3),    // 8
 };
 static const int g_num_configs = (int)(sizeof(g_configs) / sizeof(g_configs[0]));
 
@@ -540,18 +638,34 @@ static bool fast_eligible(const GemmParams& p) {
   return true;
 }
 
+// Tile choice: score = (measured relative efficiency of the tile class) x (fraction of the
+// 256 CUs kept busy over all rounds of workgroups) x (fraction of the tiles' area that is real
+// output).  Within a class the wave arrangement depends on the output width: 4-byte outputs
+// store straight from the MFMA layout and prefer waves stacked along M, int8 outputs go through
+// the LDS staging and prefer waves along N; very long K favours four fat waves over eight.
 static int pick_config(const GemmParams& p) {
   if (!fast_eligible(p)) return 0;
-  // Largest tile that still gives every CU work; measured preferences are encoded as the
-  // candidate order.
-  const int64_t cus = 256;
-  const int cand[] = {1, 5, 9};
-  for (int c : cand) {
-    const Config& k = g_configs[c];
-    const int64_t tiles = (int64_t)((p.M + k.bm - 1) / k.bm) * ((p.N + k.bn - 1) / k.bn) * p.batch;
-    if (tiles >= cus || c == 9) return c;
+  const bool wide_out = out_class(p.out_dtype) != OUT8;
+  struct Cand { int cfg; double base; };
+  const Cand cands[] = {
+      {wide_out ? 5 : 4, 1.00},
+      {wide_out ? 2 : (p.K >= 8192 ? 1 : 3), 0.93},
+      {6, 0.78},
+      {8, 0.50},
+  };
+  int best = 8;
+  double best_score = -1.0;
+  for (const Cand& c : cands) {
+    const Config& k = g_configs[c.cfg];
+    const int64_t tm = (p.M + k.bm - 1) / k.bm, tn = (p.N + k.bn - 1) / k.bn;
+    const int64_t tiles = tm * tn * p.batch;
+    const int64_t rounds = (tiles + 255) / 256;
+    const double busy = (double)tiles / (double)(rounds * 256);
+    const double area = ((double)p.M * p.N) / ((double)(tm * k.bm) * (double)(tn * k.bn));
+    const double score = c.base * busy * area;
+    if (score > best_score) best_score = score, best = c.cfg;
   }
-  return 9;
+  return best;
 }
 
 static int pick_group_m(const GemmParams& p, const Config& k) {
@@ -649,6 +763,12 @@ int ti_bmm_i8(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk, const int8
   return ti_bmm_i8_config(A, sAb, sAm, sAk, B, sBb, sBn, sBk, C, sCb, sCm, sCn, batch, M, N, K, bias, bias_kind,
                           alpha, beta, epilogue, out_dtype, round_mode, -1, stream);
 }
+
+#ifdef TI_TRACE
+int ti_debug_trace(unsigned long long* dst, int n) {
+  return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(ti::ti_trace_buf), sizeof(unsigned long long) * n);
+}
+#endif
 
 int ti_gemm_num_configs(void) { return ti::g_num_configs; }
 
