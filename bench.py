@@ -100,6 +100,24 @@ def time_region(torch, fn, iters, warm):
     return s.elapsed_time(e) / iters  # ms
 
 
+def mfma_issue_peak(torch, lib, random_operands):
+    """TOPS of back-to-back int8 MFMAs on register operands (no memory traffic) at the clock the chip
+    sustains; with random operand bytes this is the ceiling a GEMM on random int8 data can approach."""
+    import ctypes
+
+    ops = ctypes.c_double(0.0)
+    stream = torch.cuda.current_stream().cuda_stream
+    lib.ti_mfma_i8_probe(2000, random_operands, stream, ctypes.byref(ops))  # warm-up
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    rc = lib.ti_mfma_i8_probe(20000, random_operands, stream, ctypes.byref(ops))
+    e.record()
+    torch.cuda.synchronize()
+    assert rc == 0
+    return ops.value / (s.elapsed_time(e) * 1e-3) / 1e12
+
+
 def extras(torch, dev):
     """GB/s of the HBM-bound kernels at the baseline's shapes (algorithmic bytes / time)."""
     from triton_int_amd.kernels import bmm, fused
@@ -238,6 +256,11 @@ def main():
             "ops_per_launch": dom_ops / n_dom,
         },
     }
+    peak_rand = mfma_issue_peak(torch, lib, 1)
+    peak_const = mfma_issue_peak(torch, lib, 0)
+    result["roofline"]["measured_mfma_issue_peak_random_operands"] = peak_rand
+    result["roofline"]["measured_mfma_issue_peak_constant_operands"] = peak_const
+    result["roofline"]["frac_of_measured_issue_peak"] = achieved / peak_rand
     if not args.no_extra:
         result["extra"] = extras(torch, dev)
     if not args.no_cpu:

@@ -74,6 +74,16 @@ int ti_version(void);
 /* Message for the last non-zero status returned on the calling thread ("" if none). */
 const char* ti_last_error(void);
 
+/*
+ * Measurement aid, no counterpart in the reference: enqueues a kernel that issues `iters` x 8
+ * independent v_mfma_i32_32x32x32_i8 per wavefront on register operands (constant bytes, or
+ * pseudo-random bytes when random_operands != 0) with no memory traffic.  *ops_out (host, may be
+ * NULL) receives the int8 ops of the launch (2*M*N*K convention); the caller times it.  Gives
+ * the matrix-pipe rate at the clock the chip actually sustains, which a benchmark reports beside
+ * the nominal peak.
+ */
+int ti_mfma_i8_probe(int iters, int random_operands, void* stream, double* ops_out);
+
 /* ---- int8 GEMM / BMM --------------------------------------------------------------- */
 
 /*

@@ -51,11 +51,62 @@ int launch_status(const char* what) {
   return TI_OK;
 }
 
+// ---- MFMA issue-rate probe ---------------------------------------------------------------------
+// Back-to-back v_mfma_i32_32x32x32_i8 on register operands only (no LDS, no memory): the rate the
+// matrix pipes sustain at the clock the power management settles on.  With random operand bytes
+// that clock is far below the nominal one, so this, not the data-sheet peak, is the ceiling a
+// GEMM on random int8 data can approach.
+constexpr int PROBE_BLOCKS = 1024, PROBE_THREADS = 256, PROBE_ACC = 8;
+__device__ int g_probe_sink[PROBE_BLOCKS * PROBE_THREADS];
+
+__device__ __forceinline__ unsigned probe_hash(unsigned x) {
+  x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+  return x;
+}
+
+__global__ __launch_bounds__(PROBE_THREADS) void mfma_probe_kernel(int iters, int random_operands) {
+  v4i a[PROBE_ACC], b[PROBE_ACC];
+#pragma unroll
+  for (int i = 0; i < PROBE_ACC; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const unsigned s = (blockIdx.x * PROBE_THREADS + threadIdx.x) * 64u + i * 8u + j;
+      a[i][j] = random_operands ? (int)probe_hash(s) : 0x01010101;
+      b[i][j] = random_operands ? (int)probe_hash(s + 4u) : 0x02020202;
+    }
+  v16i acc[PROBE_ACC];
+#pragma unroll
+  for (int i = 0; i < PROBE_ACC; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[i][r] = 0;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < PROBE_ACC; ++i)
+      acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[i], acc[i], 0, 0, 0);
+  }
+  int s = 0;
+#pragma unroll
+  for (int i = 0; i < PROBE_ACC; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s += acc[i][r];
+  g_probe_sink[blockIdx.x * PROBE_THREADS + threadIdx.x] = s;
+}
+
 }  // namespace ti
 
 extern "C" {
 
 int ti_version(void) { return 1; }
+
+int ti_mfma_i8_probe(int iters, int random_operands, void* stream, double* ops_out) {
+  if (iters < 0) return ti::fail(TI_E_SHAPE, "negative iteration count");
+  int rc = ti::check_device();
+  if (rc != TI_OK) return rc;
+  ti::mfma_probe_kernel<<<dim3(ti::PROBE_BLOCKS), dim3(ti::PROBE_THREADS), 0, (hipStream_t)stream>>>(iters, random_operands);
+  if (ops_out)
+    *ops_out = (double)ti::PROBE_BLOCKS * (ti::PROBE_THREADS / 64) * (double)iters * ti::PROBE_ACC * 65536.0;
+  return ti::launch_status("mfma_probe_kernel");
+}
 
 const char* ti_last_error(void) { return ti::g_err; }
 
