@@ -1,0 +1,99 @@
+"""CPU-side checks: the built library exports every function the public header declares, and the
+host-side mirror of the reference interface (modules, buffers, scale algebra, argument checks)
+behaves without a GPU.  No kernel is launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    text = open(os.path.join(ROOT, "include", "triton_int_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ti_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from triton_int_amd import _lib
+    names = declared_functions()
+    assert "ti_bmm_i8" in names and "ti_layernorm_q" in names and len(names) >= 10
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, missing
+    assert set(names) == set(_lib.EXPORTS)
+    assert _lib.lib().ti_version() == 1
+    n = _lib.lib().ti_gemm_num_configs()
+    assert n >= 5 and _lib.lib().ti_gemm_config_name(0).decode().startswith("gather")
+
+
+def test_missing_library_raises(monkeypatch):
+    from triton_int_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libtriton_int_hip.so")
+    with pytest.raises(RuntimeError, match="no CPU or Triton fallback"):
+        _lib.lib()
+
+
+def test_cpu_tensors_are_refused_not_emulated():
+    from triton_int_amd.kernels.linear import linear_a8_w8_b8_o8
+    from triton_int_amd.kernels.fused import gelu_q, layer_norm_fwd_fused_single_pass_q
+    a = torch.zeros((4, 16), dtype=torch.int8)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        linear_a8_w8_b8_o8(a, a, torch.zeros(4, dtype=torch.int8), 1.0, 1.0)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        gelu_q(torch.zeros(8), 1.0)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        layer_norm_fwd_fused_single_pass_q(torch.zeros(2, 8), torch.ones(8), torch.zeros(8), 1e-5)
+    with pytest.raises(AssertionError, match="Incompatible dimensions"):
+        linear_a8_w8_b8_o8(a, torch.zeros((4, 32), dtype=torch.int8), None, 1.0, 1.0)
+
+
+def test_module_buffers_match_reference_names():
+    from triton_int_amd.nn import bmm, fused, linear
+    m = linear.W8A8B8O8Linear(32, 16, alpha=0.5, beta=0.25)
+    sd = m.state_dict()
+    assert list(sd) == ["weight", "bias", "a", "b"]
+    assert sd["weight"].shape == (16, 32) and sd["weight"].dtype == torch.int8
+    assert sd["bias"].dtype == torch.int8 and sd["a"].dtype == torch.float32 and sd["a"].ndim == 0
+    assert int(sd["weight"].min()) >= -127 and int(sd["weight"].max()) <= 126
+    assert linear.W8A8B32O32Linear(8, 8).bias.dtype == torch.int32
+    assert list(linear.W8A8B32O32LinearWithoutScaling(8, 8).state_dict()) == ["weight", "bias"]
+    assert linear.W8A8BFP32OFP32Linear(8, 8, alpha=3.0, beta=9.0).b.item() == 1.0
+    assert list(bmm.BMM_S8T_S8N_S8T(0.5).state_dict()) == ["a"]
+    ln = fused.LayerNormQ(24)
+    assert list(ln.state_dict()) == ["weight", "bias"] and ln.eps == 1e-5 and ln.input_scale == 1.0
+    assert fused.DQ_Add_LayerNorm_Q(24).input_scale == 1.0
+    # state dicts interchange: load a dict with the reference's key names
+    m2 = linear.W8A8B8O8Linear(32, 16)
+    m2.load_state_dict(sd)
+    assert torch.equal(m2.weight, m.weight) and float(m2.a) == 0.5
+
+
+def test_from_float_algebra_on_cpu():
+    from triton_int_amd.functional.quantization import (quantize_per_tensor_absmax,
+                                                        quantize_weight_per_channel_absmax,
+                                                        dynamic_quantize_activation_per_token_absmax)
+    from triton_int_amd.nn.bmm import BMM_S8T_S8N_F32T, BMM_S8T_S8N_S8T
+    from triton_int_amd.nn.linear import W8A8B32O32Linear
+    torch.manual_seed(1)
+    w = torch.randn(6, 10)
+    q, s = quantize_per_tensor_absmax(w.clone())
+    assert q.dtype == torch.int8 and torch.allclose(s, w.abs().max() / 127)
+    assert torch.equal(q, (w / s).round().to(torch.int8)) and int(q.abs().max()) == 127
+    qc, sc = quantize_weight_per_channel_absmax(w.clone())
+    assert sc.shape == (6, 1) and torch.all(qc.abs().max(dim=1)[0] == 127)
+    x = torch.randn(4, 10)
+    qa, sa = dynamic_quantize_activation_per_token_absmax(x.clone())
+    assert qa.dtype == torch.int8 and sa.shape == (4, 1)
+    assert torch.allclose(qa.float() * sa, x, atol=float(sa.max()))
+    lin = torch.nn.Linear(10, 6)
+    b0 = lin.bias.detach().clone()
+    m = W8A8B32O32Linear.from_float(lin, 0.02, 0.05)
+    bs = b0.abs().max() / (2**31 - 1)
+    assert m.bias.dtype == torch.int32 and torch.allclose(m.b, bs / 0.05)
+    assert abs(float(BMM_S8T_S8N_S8T.from_scale(0.02, 0.03, 0.6).a) - 0.001) < 1e-9
+    assert abs(float(BMM_S8T_S8N_F32T.from_scale(0.5, 0.25).a) - 0.125) < 1e-9

@@ -1,0 +1,93 @@
+"""Committed fixtures (tests/golden/*.npz, made by tests/golden/make_golden.py): the CPU test freezes
+the oracle against them; the GPU tests run the HIP kernels on the fixture inputs."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+
+G = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def load(name):
+    return dict(np.load(os.path.join(G, name), allow_pickle=False))
+
+
+def test_oracle_reproduces_fixtures():
+    d = load("gemm.npz")
+    assert np.array_equal(O.linear_a8_w8_b32_o32(d["a"], d["w"], d["b32"]), d["o32"])
+    assert np.array_equal(O.linear_a8_w8_b8_o8(d["a"], d["w"], d["b8"], d["alpha"], d["beta"]), d["o8_rne"])
+    assert np.array_equal(O.linear_a8_w8_b8_o8(d["a"], d["w"], d["b8"], d["alpha"], d["beta"], round_mode=O.TRUNC), d["o8_trunc"])
+    assert np.array_equal(O.linear_a8_w8_bfp32_ofp32_GeLu_Q(d["a"], d["w"], d["bf"], d["ag"], d["bg"]), d["gelu_rne"])
+    assert np.array_equal(O.linear_a8_w8_ofp32(d["big_a"], d["big_w"], np.float32(1.0)), d["big_of32"])
+    # hand-checkable content of the fixture: ties with alpha = 0.5 on row 1 (bias term removed)
+    acc_row = d["o32"][1, 2:18].astype(np.int64) - d["b32"][2:18]
+    assert acc_row.tolist() == list(range(-7, 9))
+    assert d["o32"][0, 0] - d["b32"][0] == 80 * 127 * 127 and d["o8_rne"][0, 0] == 127 and d["o8_rne"][0, 1] == -128
+    b = load("bmm.npz")
+    assert np.array_equal(O.bmm_s8t_s8n_s8t(b["a"], b["b"], b["alpha"]), b["s8"])
+    r = load("rows.npz")
+    for cols in (128, 768, 5120):
+        assert np.array_equal(O.layernorm_q(r[f"x{cols}"], r[f"w{cols}"], r[f"b{cols}"], 1e-5), r[f"y{cols}"])
+    assert np.array_equal(O.gelu_q(r["gelu_x"], r["gelu_scale"]), r["gelu_y"])
+    rout, q = O.dq_add_layernorm_q(r["dq_acc"], 1e-5, r["dq_res"], r["w768"], r["b768"], 1e-5)
+    assert np.array_equal(rout, r["dq_rout"]) and np.array_equal(q, r["dq_q"])
+
+
+def _dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to("cuda:0")
+
+
+def _host(t):
+    t = t.cpu()
+    return t.view(torch.int16).numpy().view(np.uint16) if t.dtype in (torch.float16, torch.bfloat16) else t.numpy()
+
+
+@pytest.mark.gpu
+def test_gpu_gemm_fixture_all_epilogues_and_configs():
+    from triton_int_amd import _lib
+    from triton_int_amd.kernels import fused, linear
+    d = load("gemm.npz")
+    a, w = _dev(d["a"]), _dev(d["w"])
+    al, be = float(d["alpha"]), float(d["beta"])
+    for cfg in range(-1, _lib.lib().ti_gemm_num_configs()):
+        assert np.array_equal(_host(linear.linear_a8_w8_b32_o32(a, w, _dev(d["b32"]), _config=cfg)), d["o32"])
+        assert np.array_equal(_host(linear.linear_a8_w8_b32_o32_with_scaling(a, w, _dev(d["b32"]), 0.01, be, _config=cfg)), d["o32_scaled"])
+        for name, rm in (("rne", 0), ("trunc", 1)):
+            assert np.array_equal(_host(linear.linear_a8_w8_b8_o8(a, w, _dev(d["b8"]), al, be, _round_mode=rm, _config=cfg)), d[f"o8_{name}"])
+            assert np.array_equal(_host(linear.linear_relu_a8_w8_b8_o8(a, w, _dev(d["b8"]), al, be, _round_mode=rm, _config=cfg)), d[f"o8_relu_{name}"])
+            got = _host(fused.linear_a8_w8_bfp32_ofp32_GeLu_Q(a, w, _dev(d["bf"]), float(d["ag"]), float(d["bg"]), _round_mode=rm, _config=cfg))
+            diff = np.abs(got.astype(int) - d[f"gelu_{name}"].astype(int))
+            assert diff.max() <= 1 and (diff != 0).mean() < 1e-3
+        assert np.array_equal(_host(linear.linear_a8_w8_bfp32_ofp32(a, w, _dev(d["bf"]), 0.0037, 1.0, _config=cfg)), d["of32"])
+        assert np.array_equal(_host(linear.linear_a8_w8_bfp32_ofp32(a, w, _dev(d["bf"]), 0.0037, 1.0, dtype=torch.float16, _config=cfg)), d["of16"])
+        assert np.array_equal(_host(linear.linear_a8_w8_bfp32_ofp32(a, w, _dev(d["bf"]), 0.0037, 1.0, dtype=torch.bfloat16, _config=cfg)), d["obf16"])
+        assert np.array_equal(_host(linear.linear_a8_w8_b32_o32(_dev(d["big_a"]), _dev(d["big_w"]), None, _config=cfg)), d["big_o32"])
+        assert np.array_equal(_host(linear.linear_a8_w8_ofp32(_dev(d["big_a"]), _dev(d["big_w"]), 1.0, _config=cfg)), d["big_of32"])
+
+
+@pytest.mark.gpu
+def test_gpu_bmm_and_rows_fixtures():
+    from triton_int_amd.kernels import bmm, fused
+    b = load("bmm.npz")
+    a, bb = _dev(b["a"]), _dev(b["b"])
+    assert np.array_equal(_host(bmm.bmm_s8t_s8n_s32t(a, bb)), b["s32"])
+    assert np.array_equal(_host(bmm.bmm_s8t_s8n_s8t(a, bb, float(b["alpha"]))), b["s8"])
+    assert np.array_equal(_host(bmm.bmm_s8t_s8n_f32t(a, bb, float(b["alpha"]))), b["f32"])
+    assert np.array_equal(_host(bmm.bmm_s8t_s8t_s8t(a, bb.transpose(1, 2).contiguous(), float(b["alpha"]))), b["s8"])
+    r = load("rows.npz")
+    for cols in (128, 768, 5120):
+        y, mean, rstd = fused.layer_norm_fwd_fused_single_pass_q(_dev(r[f"x{cols}"]), _dev(r[f"w{cols}"]), _dev(r[f"b{cols}"]), 1e-5, _return_stats=True)
+        diff = np.abs(_host(y).astype(int) - r[f"y{cols}"].astype(int))
+        assert diff.max() <= 1 and (diff != 0).mean() < 1e-3
+        assert np.allclose(_host(mean), r[f"mean{cols}"], atol=1e-4 * max(1.0, float(np.abs(r[f"mean{cols}"]).max())))
+        assert np.allclose(_host(rstd)[2:], r[f"rstd{cols}"][2:], rtol=1e-4)
+    rout, q = fused.dq_add_layernorm_q(_dev(r["dq_acc"]), 1e-5, _dev(r["dq_res"]), _dev(r["w768"]), _dev(r["b768"]), 1e-5)
+    assert np.array_equal(_host(rout), r["dq_rout"])
+    diff = np.abs(_host(q).astype(int) - r["dq_q"].astype(int))
+    assert diff.max() <= 1 and (diff != 0).mean() < 1e-3
+    y = _host(fused.gelu_q(_dev(r["gelu_x"]), float(r["gelu_scale"])))
+    diff = np.abs(y.astype(int) - r["gelu_y"].astype(int))
+    assert diff.max() <= 1 and (diff != 0).mean() < 2e-3
