@@ -607,8 +607,8 @@ static const Config g_configs[] = {
     TI_FAST(256, 128, 128, 2, 2, 1, 3),  // 1
     TI_FAST(256, 128, 128, 4, 2, 1, 3),  // 2
     TI_FAST(256, 128, 128, 2, 4, 1, 3),  // 3
-    TI_FAST(256, 256, 64, 2, 4, 2, 3),   // 4
-    TI_FAST(256, 256, 64, 4, 2, 2, 3),   // 5
+    TI_FAST(256, 256, 64, 2, 4, 2, 4),   // 4
+    TI_FAST(256, 256, 64, 4, 2, 2, 4),   // 5
     TI_FAST(128, 128, 64, 2, 2, 2, 4),   // 6
     TI_FAST(128, 128, 128, 2, 2, 1, 3),  // 7
     TI_FAST(64, 64, 128, 2, 2, 1, 3),    // 8
@@ -642,14 +642,14 @@ static bool fast_eligible(const GemmParams& p) {
 // 256 CUs kept busy over all rounds of workgroups) x (fraction of the tiles' area that is real
 // output).  Within a class the wave arrangement depends on the output width: 4-byte outputs
 // store straight from the MFMA layout and prefer waves stacked along M, int8 outputs go through
-// the LDS staging and prefer waves along N; very long K favours four fat waves over eight.
+// the LDS staging; the preferences were measured with weights streamed from HBM.
 static int pick_config(const GemmParams& p) {
   if (!fast_eligible(p)) return 0;
   const bool wide_out = out_class(p.out_dtype) != OUT8;
   struct Cand { int cfg; double base; };
   const Cand cands[] = {
       {wide_out ? 5 : 4, 1.00},
-      {wide_out ? 2 : (p.K >= 8192 ? 1 : 3), 0.93},
+      {wide_out ? 2 : (p.epilogue == TI_EPI_GELU_I8 ? 3 : 1), 0.90},
       {6, 0.78},
       {8, 0.50},
   };
