@@ -15,9 +15,11 @@
  *   acc      exact int32  sum_k a[m,k] * b[n,k]
  *   f(.)     int32 -> fp32 conversion, round-to-nearest-even
  *   all fp32 products and sums are separately rounded (no FMA contraction)
- *   q8(v)    TI_ROUND_RNE_CLAMP: clamp(round_half_even(v), -128, 127), NaN -> 0
+ *   q8(v)    TI_ROUND_RNE_CLAMP: clamp(round_half_even(v), -128, 127)
  *            TI_ROUND_TRUNC    : clamp(trunc(v), -128, 127)  (literal Triton `.to(int8)`
- *                                on in-range values; test-time switch only)
+ *                                on in-range values; test-time switch only, always served by
+ *                                the slow gather kernel)
+ *            The result for a NaN v (possible only with non-finite scales) is unspecified.
  */
 #ifndef TRITON_INT_HIP_H
 #define TRITON_INT_HIP_H

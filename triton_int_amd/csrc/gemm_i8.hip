@@ -408,44 +408,57 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmPa
   const EpiCtx e = make_epi(p);
   char* Cb = (char*)p.C;
   const int lrow = lane & 31, lhi = lane >> 5;
-  const bool trunc = e.round_mode == TI_ROUND_TRUNC;
   const bool has_bias = e.bias_kind != TI_BIAS_NONE;
 
   if constexpr (OUTCLS == OUT8) {
     // acc[i][j][r]: m = m0 + wm*WTM + i*32 + lrow;  n = n0 + wn*WTN + j*32 + 8*(r/4) + 4*lhi + r%4.
     // Quantise, pack 4 consecutive n into a dword, stage the tile in LDS, then write rows with
     // 16-byte stores.  (The K loop ended with a barrier, so the operand stages are free.)
-    const int q_floor = e.epilogue == TI_EPI_SCALE_RELU_I8 ? 0 : -128;  // ReLU = clamp from below at 0
-    auto body = [&](auto gelu_tag) {
+    // Per element: cvt, mul, (add), clamp in fp32 (v_med3_f32), then one add of 1.5*2^23: that
+    // add rounds to the nearest integer, ties to even, and leaves the two's-complement int8 in the
+    // low byte of the float's bit pattern.  Clamping first keeps the sum in the exact range; since
+    // the bounds are integers, clamp-then-round equals round-then-clamp.  ReLU is a lower bound of 0.
+    // (Truncation, the test-time rounding switch, is served by the gather kernel instead.)
+    const float q_floor = e.epilogue == TI_EPI_SCALE_RELU_I8 ? 0.0f : -128.0f;
+    auto body = [&](auto gelu_tag, auto bias_tag) {
       constexpr bool GELU = decltype(gelu_tag)::value;
-      auto one = [&](int a, float col) -> int {
+      constexpr bool BIAS = decltype(bias_tag)::value;
+      auto one = [&](int a, float col) -> unsigned {
         float v = (float)a * e.alpha;
-        v = col + v;  // col is 0 without a bias; adding it cannot change the quantised value
+        if constexpr (BIAS) v = col + v;
         if constexpr (GELU) v = gelu_tanh_scaled(v, e.beta);
-        const float r = trunc ? v : __builtin_rintf(v);
-        return min(max((int)r, q_floor), 127);
+        v = __builtin_amdgcn_fmed3f(v, q_floor, 127.0f);
+        return __float_as_uint(v + 12582912.0f);
       };
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const int nl = wn * WTN + j * 32 + 8 * g + 4 * lhi;
-          float col[4];
+          float col[4] = {0.f, 0.f, 0.f, 0.f};
+          if constexpr (BIAS) {
 #pragma unroll
-          for (int t = 0; t < 4; ++t)
-            col[t] = column_term_t<GELU ? TI_BIAS_F32 : TI_BIAS_I8>(e, min(n0 + nl + t, p.N - 1), GELU);
+            for (int t = 0; t < 4; ++t)
+              col[t] = column_term_t<GELU ? TI_BIAS_F32 : TI_BIAS_I8>(e, min(n0 + nl + t, p.N - 1), GELU);
+          }
 #pragma unroll
           for (int i = 0; i < TM; ++i) {
             const int ml = wm * WTM + i * 32 + lrow;
-            const unsigned w = pack4(one(acc[i][j][4 * g + 0], col[0]), one(acc[i][j][4 * g + 1], col[1]),
-                                     one(acc[i][j][4 * g + 2], col[2]), one(acc[i][j][4 * g + 3], col[3]));
-            *(unsigned*)(lds + ml * C_PITCH + nl) = w;
+            const unsigned b0 = one(acc[i][j][4 * g + 0], col[0]), b1 = one(acc[i][j][4 * g + 1], col[1]);
+            const unsigned b2 = one(acc[i][j][4 * g + 2], col[2]), b3 = one(acc[i][j][4 * g + 3], col[3]);
+            // low bytes of b0..b3 -> one dword
+            const unsigned lo = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u);
+            const unsigned hi = __builtin_amdgcn_perm(b3, b2, 0x04000c0cu);
+            *(unsigned*)(lds + ml * C_PITCH + nl) = lo | hi;
           }
         }
       }
     };
-    if (e.epilogue == TI_EPI_GELU_I8) body(std::true_type{});
-    else body(std::false_type{});
+    const bool gelu = e.epilogue == TI_EPI_GELU_I8;
+    if (gelu && has_bias) body(std::true_type{}, std::true_type{});
+    else if (gelu) body(std::true_type{}, std::false_type{});
+    else if (has_bias) body(std::false_type{}, std::true_type{});
+    else body(std::false_type{}, std::false_type{});
     __syncthreads();
     int8_t* Cz = (int8_t*)Cb + (int64_t)bz * p.sCb;
     const bool vec_ok = ((p.sCm & 15) == 0) && ((((uintptr_t)Cz) & 15) == 0);
@@ -721,9 +734,13 @@ static int run(GemmParams p, int config, hipStream_t stream) {
   rc = check_device();
   if (rc != TI_OK) return rc;
   if (!p.bias) p.bias_kind = TI_BIAS_NONE;
-  if (config < 0) config = pick_config(p);
+  // the fast kernels quantise to int8 with round-half-even only; the truncating test switch runs
+  // on the gather kernel
+  const bool trunc8 = p.round_mode == TI_ROUND_TRUNC && out_class(p.out_dtype) == OUT8;
+  if (config < 0) config = trunc8 ? 0 : pick_config(p);
   if (config >= g_num_configs) return fail(TI_E_COMBO, "config %d out of range", config);
   const Config& k = g_configs[config];
+  if (k.fast && trunc8) return fail(TI_E_COMBO, "config %s does not implement TI_ROUND_TRUNC for int8 outputs", k.name);
   if (k.fast && !fast_eligible(p)) return fail(TI_E_COMBO, "config %s needs K-contiguous 16-byte aligned operands", k.name);
   p.tiles_m = (p.M + k.bm - 1) / k.bm;
   p.tiles_n = (p.N + k.bn - 1) / k.bn;

@@ -70,8 +70,9 @@ __global__ __launch_bounds__(RN_THREADS) void rownorm_vec_kernel(RowNormParams p
     const int v = tid + j * RN_THREADS;
     if (v < nvec) {
       if constexpr (DQ) {
-        const v4i a = *(const v4i*)(p.acc + (int64_t)row * p.acc_rs + v * 4);
-        const v4f r = *(const v4f*)(p.resid_in + (int64_t)row * p.rin_rs + v * 4);
+        // streamed once: non-temporal, so the rows do not displace gamma/beta in the caches
+        const v4i a = __builtin_nontemporal_load((const v4i*)(p.acc + (int64_t)row * p.acc_rs + v * 4));
+        const v4f r = __builtin_nontemporal_load((const v4f*)(p.resid_in + (int64_t)row * p.rin_rs + v * 4));
         v4f o;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
@@ -80,9 +81,9 @@ __global__ __launch_bounds__(RN_THREADS) void rownorm_vec_kernel(RowNormParams p
           o[t] = r[t] + prod;
         }
         x[j] = o;
-        *(v4f*)(p.resid_out + (int64_t)row * p.rout_rs + v * 4) = o;
+        __builtin_nontemporal_store(o, (v4f*)(p.resid_out + (int64_t)row * p.rout_rs + v * 4));
       } else {
-        x[j] = *(const v4f*)(p.x + (int64_t)row * p.x_rs + v * 4);
+        x[j] = __builtin_nontemporal_load((const v4f*)(p.x + (int64_t)row * p.x_rs + v * 4));
       }
     } else {
       x[j] = (v4f){0.f, 0.f, 0.f, 0.f};
@@ -125,13 +126,13 @@ __global__ __launch_bounds__(RN_THREADS) void rownorm_vec_kernel(RowNormParams p
       v4f o;
 #pragma unroll
       for (int t = 0; t < 4; ++t) o[t] = norm_one(x[j][t], mean, rstd, w[t], b[t], has_b);
-      if (p.ln_out) *(v4f*)(p.ln_out + (int64_t)row * p.ln_rs + v * 4) = o;
+      if (p.ln_out) __builtin_nontemporal_store(o, (v4f*)(p.ln_out + (int64_t)row * p.ln_rs + v * 4));
       if (p.y) {
         const int q0 = q8(o[0], p.round_mode), q1 = q8(o[1], p.round_mode), q2 = q8(o[2], p.round_mode),
                   q3 = q8(o[3], p.round_mode);
         int8_t* dst = p.y + (int64_t)row * p.y_rs + v * 4;
         if (y_vec) {
-          *(unsigned*)dst = pack4(q0, q1, q2, q3);
+          __builtin_nontemporal_store(pack4(q0, q1, q2, q3), (unsigned*)dst);
         } else {
           dst[0] = (int8_t)q0; dst[1] = (int8_t)q1; dst[2] = (int8_t)q2; dst[3] = (int8_t)q3;
         }
@@ -221,28 +222,28 @@ static int launch_rownorm(const RowNormParams& p, hipStream_t stream) {
 constexpr int GQ_THREADS = 256;
 constexpr int GQ_UNROLL = 4;
 
+// Each workgroup converts one contiguous run of GQ_UNROLL * 256 float4 vectors (16 KB in, 4 KB
+// out): every load instruction of a wave covers 1 KB, every store 256 B, all loads are issued
+// before the first use, and the streams bypass the caches (non-temporal).
 __global__ __launch_bounds__(GQ_THREADS) void gelu_q_vec_kernel(const float* __restrict__ x, const float* scale,
                                                                 int8_t* __restrict__ y, int64_t nvec,
                                                                 int round_mode) {
   const float s = *scale;
-  const int64_t stride = (int64_t)gridDim.x * GQ_THREADS;
-  int64_t v = (int64_t)blockIdx.x * GQ_THREADS + threadIdx.x;
-  for (; v + (GQ_UNROLL - 1) * stride < nvec; v += GQ_UNROLL * stride) {
-    v4f in[GQ_UNROLL];
+  const int64_t base = (int64_t)blockIdx.x * (GQ_THREADS * GQ_UNROLL) + threadIdx.x;
+  v4f in[GQ_UNROLL];
 #pragma unroll
-    for (int u = 0; u < GQ_UNROLL; ++u) in[u] = *(const v4f*)(x + (v + u * stride) * 4);
+  for (int u = 0; u < GQ_UNROLL; ++u) {
+    const int64_t v = base + u * GQ_THREADS;
+    if (v < nvec) in[u] = __builtin_nontemporal_load((const v4f*)x + v);
+  }
 #pragma unroll
-    for (int u = 0; u < GQ_UNROLL; ++u) {
+  for (int u = 0; u < GQ_UNROLL; ++u) {
+    const int64_t v = base + u * GQ_THREADS;
+    if (v < nvec) {
       const unsigned w = pack4(q8(gelu_tanh_scaled(in[u][0], s), round_mode), q8(gelu_tanh_scaled(in[u][1], s), round_mode),
                                q8(gelu_tanh_scaled(in[u][2], s), round_mode), q8(gelu_tanh_scaled(in[u][3], s), round_mode));
-      *(unsigned*)(y + (v + u * stride) * 4) = w;
+      __builtin_nontemporal_store(w, (unsigned*)y + v);
     }
-  }
-  for (; v < nvec; v += stride) {
-    const v4f in = *(const v4f*)(x + v * 4);
-    const unsigned w = pack4(q8(gelu_tanh_scaled(in[0], s), round_mode), q8(gelu_tanh_scaled(in[1], s), round_mode),
-                             q8(gelu_tanh_scaled(in[2], s), round_mode), q8(gelu_tanh_scaled(in[3], s), round_mode));
-    *(unsigned*)(y + v * 4) = w;
   }
 }
 
@@ -307,8 +308,8 @@ int ti_gelu_q(const float* x, const float* scale, int8_t* y, int64_t n, int roun
   int64_t done = 0;
   if ((((uintptr_t)x) & 15) == 0 && (((uintptr_t)y) & 3) == 0 && n >= 4) {
     const int64_t nvec = n / 4;
-    int64_t blocks = (nvec + ti::GQ_THREADS * ti::GQ_UNROLL - 1) / (ti::GQ_THREADS * ti::GQ_UNROLL);
-    if (blocks > 256 * 16) blocks = 256 * 16;
+    const int64_t blocks = (nvec + ti::GQ_THREADS * ti::GQ_UNROLL - 1) / (ti::GQ_THREADS * ti::GQ_UNROLL);
+    if (blocks > 0x7fffffff) return ti::fail(TI_E_SHAPE, "n too large");
     ti::gelu_q_vec_kernel<<<dim3((unsigned)blocks), dim3(ti::GQ_THREADS), 0, s>>>(x, scale, y, nvec, round_mode);
     rc = ti::launch_status("gelu_q_vec_kernel");
     if (rc != TI_OK) return rc;
