@@ -16,10 +16,14 @@ def _lib():
     return L
 
 
-def _configs():
+def _configs(M=1):
+    """(index, name) of every kernel configuration that can run M activation rows"""
     L = _lib()
     n = L.lib().ti_gemm_num_configs()
-    return [(i, L.lib().ti_gemm_config_name(i).decode()) for i in range(n)]
+    out = [(i, L.lib().ti_gemm_config_name(i).decode()) for i in range(n)]
+    def fits(nm):  # "skinny_m<rows>_..." configurations take at most <rows> activation rows
+        return not nm.startswith("skinny") or M <= int(nm.split("_")[1][1:])
+    return [(i, nm) for i, nm in out if fits(nm)]
 
 
 def _kl():
@@ -40,7 +44,7 @@ def test_all_configs_int32_bit_exact(shape):
     bias = g.integers(-2**24, 2**24, size=N, dtype=np.int32)
     want = O.linear_a8_w8_b32_o32(a, w, bias)
     ga, gw, gb = gpu(a), gpu(w), gpu(bias)
-    for cfg, name in _configs():
+    for cfg, name in _configs(M):
         got = cpu(linear.linear_a8_w8_b32_o32(ga, gw, gb, _config=cfg))
         assert np.array_equal(got, want), f"config {name}"
     got = cpu(linear.linear_a8_w8_b32_o32(ga, gw, gb))
@@ -59,7 +63,7 @@ def test_all_configs_int8_epilogues_bit_exact(shape):
         want = O.linear_a8_w8_b8_o8(a, w, bias, alpha, beta)
         want_relu = O.linear_relu_a8_w8_b8_o8(a, w, bias, alpha, beta)
         want_tr = O.linear_a8_w8_b8_o8(a, w, bias, alpha, beta, round_mode=O.TRUNC)
-        for cfg, name in _configs():
+        for cfg, name in _configs(M):
             got = cpu(linear.linear_a8_w8_b8_o8(ga, gw, gb, alpha, beta, _config=cfg))
             assert np.array_equal(got, want), f"o8 config {name} alpha {alpha}"
             got = cpu(linear.linear_relu_a8_w8_b8_o8(ga, gw, gb, alpha, beta, _config=cfg))
@@ -85,7 +89,7 @@ def test_all_configs_float_and_scaled_i32(shape):
     want_b = O.linear_a8_w8_bfp32_ofp32(a, w, bias_f, alpha, beta, out_dtype=O.DT_BF16)
     want_nb = O.linear_a8_w8_ofp32(a, w, alpha)
     want_s = O.linear_a8_w8_b32_o32_with_scaling(a, w, bias_i, alpha, beta)
-    for cfg, name in _configs():
+    for cfg, name in _configs(M):
         got = cpu(linear.linear_a8_w8_bfp32_ofp32(ga, gw, gpu(bias_f), alpha, beta, _config=cfg))
         assert got.dtype == np.float32 and np.array_equal(got, want_f), f"f32 {name}"
         got = cpu(linear.linear_a8_w8_bfp32_ofp32(ga, gw, gpu(bias_f), alpha, beta, dtype=torch.float16, _config=cfg))
@@ -110,7 +114,7 @@ def test_all_configs_gelu_q(shape):
     want = O.linear_a8_w8_bfp32_ofp32_GeLu_Q(a, w, bias, alpha, beta)
     assert np.unique(want).size > 100  # the case really exercises the rounding, not only the clamp
     ga, gw, gb = gpu(a), gpu(w), gpu(bias)
-    for cfg, name in _configs():
+    for cfg, name in _configs(M):
         got = cpu(fused.linear_a8_w8_bfp32_ofp32_GeLu_Q(ga, gw, gb, alpha, beta, _config=cfg))
         mx, rate = mismatch_report(got, want)
         assert mx <= 1 and rate < 1e-3, f"{name}: max {mx} rate {rate}"
@@ -166,7 +170,7 @@ def test_bmm_fast_path_all_configs(B, M, N, K):
     alpha = np.float32(1e-3)
     want8 = O.bmm_s8t_s8n_s8t(a, b, alpha)
     wantf = O.bmm_s8t_s8n_f32t(a, b, alpha)
-    for cfg, name in _configs():
+    for cfg, name in _configs(M):
         assert np.array_equal(cpu(bmm.bmm_s8t_s8n_s32t(ga, gb, _config=cfg)), want32), name
         assert np.array_equal(cpu(bmm.bmm_s8t_s8n_s8t(ga, gb, alpha, _config=cfg)), want8), name
         assert np.array_equal(cpu(bmm.bmm_s8t_s8n_f32t(ga, gb, alpha, _config=cfg)), wantf), name
@@ -275,3 +279,43 @@ def test_baseline_config2_opt67b_shapes_sampled_rows(which):
     s = cpu(linear.linear_a8_w8_b32_o32(gpu((x1 + x2).astype(np.int8)), gw, None))
     p1 = cpu(linear.linear_a8_w8_b32_o32(gpu(x1), gw, None)); p2 = cpu(linear.linear_a8_w8_b32_o32(gpu(x2), gw, None))
     assert np.array_equal(s, p1 + p2)
+
+
+@pytest.mark.parametrize("M,N,K", [(16, 5120, 5120), (1, 5120, 5120), (17, 272, 1040), (48, 100, 64), (64, 20480, 5120), (16, 5120, 20480)])
+def test_decode_shapes_skinny_kernel(M, N, K):
+    """M <= 64 takes the weight-streaming kernel (K split across waves, int32 partials added in LDS)."""
+    linear, _, fused = _kl()
+    L = _lib()
+    g = rng(M * 13 + N)
+    a, w = rand_i8(g, M, K, lo=-128), rand_i8(g, N, K, lo=-128)
+    b32 = g.integers(-2**20, 2**20, size=N, dtype=np.int32)
+    b8 = rand_i8(g, N); bf = g.standard_normal(N).astype(np.float32)
+    ga, gw = gpu(a), gpu(w)
+    got = cpu(linear.linear_a8_w8_b32_o32(ga, gw, gpu(b32)))
+    assert L.lib().ti_gemm_config_name(L.lib().ti_gemm_last_config()).decode().startswith("skinny")
+    assert np.array_equal(got, O.linear_a8_w8_b32_o32(a, w, b32))
+    alpha = np.float32(40.0 / (np.sqrt(K) * 127 * 127 / 3)); beta = np.float32(0.05)
+    assert np.array_equal(cpu(linear.linear_a8_w8_b8_o8(ga, gw, gpu(b8), alpha, beta)), O.linear_a8_w8_b8_o8(a, w, b8, alpha, beta))
+    assert np.array_equal(cpu(linear.linear_a8_w8_b8_o8(ga, gw, gpu(b8), alpha, beta, _round_mode=1)),
+                          O.linear_a8_w8_b8_o8(a, w, b8, alpha, beta, round_mode=O.TRUNC))
+    assert np.array_equal(cpu(linear.linear_relu_a8_w8_b8_o8(ga, gw, gpu(b8), alpha, beta)), O.linear_relu_a8_w8_b8_o8(a, w, b8, alpha, beta))
+    assert np.array_equal(cpu(linear.linear_a8_w8_bfp32_ofp32(ga, gw, gpu(bf), alpha, 1.0)), O.linear_a8_w8_bfp32_ofp32(a, w, bf, alpha, 1.0))
+    ag = np.float32(3.0 / (np.sqrt(K) * 127 * 127 / 3))
+    mx, rate = mismatch_report(cpu(fused.linear_a8_w8_bfp32_ofp32_GeLu_Q(ga, gw, gpu(bf), ag, 20.0)),
+                               O.linear_a8_w8_bfp32_ofp32_GeLu_Q(a, w, bf, ag, np.float32(20.0)))
+    assert mx <= 1 and rate < 1e-3
+
+
+def test_decode_attention_bmms():
+    """16 query tokens against a 2048-long int8 KV, 40 heads of 128 (OPT-13B decode)."""
+    _, bmm, _ = _kl()
+    g = rng(99)
+    H, T, S, D = 40, 16, 2048, 128
+    q, k = rand_i8(g, H, T, D), rand_i8(g, H, S, D)
+    sc = bmm.bmm_s8t_s8n_s8t(gpu(q), gpu(k), 1e-3)
+    assert sc.shape == (H, T, S)
+    assert np.array_equal(cpu(sc), O.bmm_s8t_s8n_s8t(q, k, np.float32(1e-3)))
+    pr = rand_i8(g, H, T, S, lo=0, hi=127); vt = rand_i8(g, H, D, S)
+    out = bmm.bmm_s8t_s8n_f32t(gpu(pr), gpu(vt), 1.0 / 16129)
+    assert np.array_equal(cpu(out), O.bmm_s8t_s8n_f32t(pr, vt, np.float32(1.0 / 16129)))
+    assert np.array_equal(cpu(bmm.bmm_s8t_s8n_s32t(gpu(pr), gpu(vt))), O.bmm_s8t_s8n_s32t(pr, vt))

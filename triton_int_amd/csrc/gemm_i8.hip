@@ -29,6 +29,7 @@ struct GemmParams {
   const float* beta;
   int epilogue, out_dtype, round_mode;
   int tiles_m, tiles_n, group_m;
+  int ksplit;  // skinny kernel: waves of a workgroup that share one 16-row slab and split K
 };
 
 enum OutClass { OUT8 = 0, OUT32 = 1, OUT16 = 2 };
@@ -595,6 +596,140 @@ __global__ __launch_bounds__(256) void gemm_gather_kernel(GemmParams p) {
   }
 }
 
+// ---- skinny family: M <= 64 (decode-shaped) ------------------------------------------------------
+// With a handful of activation rows the GEMM is a stream over the weight matrix: every byte of B
+// is read once and the matrix pipes idle.  Each wave owns a 16-row slab of B and, per 64-byte
+// k-step, feeds it as the row operand of v_mfma_i32_16x16x64_i8 against up to four 16-row blocks
+// of A (the 16 x 16 result block has rows = n, columns = m).  Operands go from global memory
+// straight into registers in MFMA layout (lane = row + 16 * chunk); A is tiny and stays in L2.
+// The 8 waves of a workgroup either take 8 different slabs (short K) or split K between them
+// (k-steps interleaved, so that together they read consecutive bytes of a row) and add their
+// int32 partial sums through LDS — integer addition, so the result does not depend on the split.
+template <int OUTCLS, int MBMAX>
+__global__ __launch_bounds__(512) void gemm_skinny_kernel(GemmParams p) {
+  constexpr int NW = 8;
+  constexpr int U = 8 / MBMAX;  // k-steps per batch of loads; two batches are in flight
+  __shared__ int red[NW][MBMAX][256];
+  const int tid = threadIdx.x, lane = tid & 63;
+  // The wave index must be known to be wave-uniform: the trip counts below depend on it, and a
+  // branch the compiler believes divergent would wrap MFMAs in EXEC masking, which MFMAs ignore.
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ksplit = p.ksplit;
+  const int slab = blockIdx.x * (NW / ksplit) + wave / ksplit;
+  const int kpart = wave % ksplit;
+  const int bz = blockIdx.y;
+  const int MB = (p.M + 15) >> 4;
+  const int r16 = lane & 15, c4 = lane >> 4;
+  const int8_t* Ab = p.A + (int64_t)bz * p.sAb;
+  const int8_t* Bb = p.B + (int64_t)bz * p.sBb;
+  const int n_row = min(slab * 16 + r16, p.N - 1);
+  const int8_t* wrow = Bb + (int64_t)n_row * p.sBn + c4 * 16;
+  const int8_t* xrow[MBMAX];
+#pragma unroll
+  for (int mb = 0; mb < MBMAX; ++mb) xrow[mb] = Ab + (int64_t)min(mb * 16 + r16, p.M - 1) * p.sAm + c4 * 16;
+
+  v4i acc[MBMAX];
+#pragma unroll
+  for (int mb = 0; mb < MBMAX; ++mb) acc[mb] = (v4i){0, 0, 0, 0};
+
+  // This wave's k-steps are kpart, kpart + ksplit, ...  Whole 64-byte k-steps run in batches of U
+  // with two register sets: the loads of batch b+1 are issued before the MFMAs of batch b, so a
+  // wave keeps up to 2*U weight loads (1 KB each) in flight, and nothing in the batch loop looks
+  // at a loaded value before the MFMAs do.  Left-over k-steps and a K tail (K % 64 != 0, the only
+  // place that needs zero fill) are handled one at a time afterwards.  The weight stream bypasses
+  // the caches (non-temporal); A is re-read by every slab and is served by L2.
+  const int KSF = p.K >> 6;  // whole k-steps
+  const int nj = kpart < KSF ? (KSF - kpart + ksplit - 1) / ksplit : 0;
+  const int nb = nj / U;
+  const int kstride = ksplit * 64;
+  v4i wf[2][U], xf[2][U][MBMAX];
+  auto load_batch = [&](int buf, int b) {
+    const int k0 = (kpart + b * U * ksplit) * 64;
+#pragma unroll
+    for (int u = 0; u < U; ++u) wf[buf][u] = *(const v4i*)(wrow + k0 + u * kstride);
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int mb = 0; mb < MBMAX; ++mb) xf[buf][u][mb] = *(const v4i*)(xrow[mb] + k0 + u * kstride);
+  };
+  auto compute = [&](int buf) {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int mb = 0; mb < MBMAX; ++mb)
+        acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[buf][u], xf[buf][u][mb], acc[mb], 0, 0, 0);
+  };
+  if (nb > 0) load_batch(0, 0);
+  for (int b = 0; b < nb; b += 2) {
+    if (b + 1 < nb) load_batch(1, b + 1);
+    compute(0);
+    if (b + 1 >= nb) break;
+    if (b + 2 < nb) load_batch(0, b + 2);
+    compute(1);
+  }
+  // left-over whole k-steps (fewer than U): one more batch, loads first, guarded by wave-uniform tests
+  const int rem = nj - nb * U;
+  if (rem > 0) {
+    const int k0 = (kpart + nb * U * ksplit) * 64;
+#pragma unroll
+    for (int u = 0; u < U - 1; ++u)
+      if (u < rem) wf[0][u] = *(const v4i*)(wrow + k0 + u * kstride);
+#pragma unroll
+    for (int u = 0; u < U - 1; ++u)
+      if (u < rem) {
+#pragma unroll
+        for (int mb = 0; mb < MBMAX; ++mb) xf[0][u][mb] = *(const v4i*)(xrow[mb] + k0 + u * kstride);
+      }
+#pragma unroll
+    for (int u = 0; u < U - 1; ++u)
+      if (u < rem) {
+#pragma unroll
+        for (int mb = 0; mb < MBMAX; ++mb)
+          acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[0][u], xf[0][u][mb], acc[mb], 0, 0, 0);
+      }
+  }
+  if ((p.K & 63) && kpart == KSF % ksplit) {
+    const int k0 = KSF * 64;
+    const bool ok = k0 + c4 * 16 < p.K;  // K is a multiple of 16: a chunk is all in or all out
+    v4i w1 = *(const v4i*)(wrow + (ok ? k0 : 0));
+    if (!ok) w1 = (v4i){0, 0, 0, 0};
+#pragma unroll
+    for (int mb = 0; mb < MBMAX; ++mb)
+      acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, *(const v4i*)(xrow[mb] + (ok ? k0 : 0)), acc[mb], 0, 0, 0);
+  }
+
+  if (ksplit > 1) {
+#pragma unroll
+    for (int mb = 0; mb < MBMAX; ++mb)
+      if (mb < MB) *(v4i*)&red[wave][mb][lane * 4] = acc[mb];
+    __syncthreads();
+    if (kpart != 0) return;
+#pragma unroll
+    for (int mb = 0; mb < MBMAX; ++mb)
+      if (mb < MB)
+        for (int kp = 1; kp < ksplit; ++kp) acc[mb] += *(const v4i*)&red[wave + kp][mb][lane * 4];
+  }
+  if (slab * 16 >= p.N) return;
+
+  // acc[mb][i]: n = slab*16 + 4*c4 + i, m = mb*16 + r16
+  const EpiCtx e = make_epi(p);
+  constexpr int ESZ = OUTCLS == OUT8 ? 1 : (OUTCLS == OUT32 ? 4 : 2);
+  char* Cz = (char*)p.C + (int64_t)bz * p.sCb * ESZ;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int n = slab * 16 + 4 * c4 + i;
+    if (n >= p.N) continue;
+    const float col = column_term(e, n);
+    const int bias_i32 = (e.epilogue == TI_EPI_I32 && e.bias_kind == TI_BIAS_I32) ? ((const int*)e.bias)[n] : 0;
+#pragma unroll
+    for (int mb = 0; mb < MBMAX; ++mb) {
+      const int m = mb * 16 + r16;
+      if (mb < MB && m < p.M)
+        store_one<OUTCLS>(e, Cz, (int64_t)m * p.sCm + (int64_t)n * p.sCn, acc[mb][i], col, bias_i32, p.out_dtype);
+    }
+  }
+}
+
 // ---- host side ---------------------------------------------------------------------------------
 
 typedef void (*KernelFn)(GemmParams);
@@ -604,6 +739,7 @@ struct Config {
   KernelFn fn[3];  // by OutClass
   int bm, bn, bk, threads;
   bool fast;       // needs the aligned K-contiguous layout
+  bool skinny = false;  // gemm_skinny_kernel: M <= 64, grid over 16-row slabs of B
 };
 
 #define TI_FAST(BM, BN, BK, WM, WN, SWZ, NS)                                              \
@@ -625,7 +761,11 @@ static const Config g_configs[] = {
     TI_FAST(128, 128, 64, 2, 2, 2, 4),   // 6
     TI_FAST(128, 128, 128, 2, 2, 1, 3),  // 7
     TI_FAST(64, 64, 128, 2, 2, 1, 3),    // 8
+    {"skinny_m16_slab16", {gemm_skinny_kernel<OUT8, 1>, gemm_skinny_kernel<OUT32, 1>, gemm_skinny_kernel<OUT16, 1>}, 16, 16, 64, 512, true, true},  // 9
+    {"skinny_m32_slab16", {gemm_skinny_kernel<OUT8, 2>, gemm_skinny_kernel<OUT32, 2>, gemm_skinny_kernel<OUT16, 2>}, 32, 16, 64, 512, true, true},  // 10
+    {"skinny_m64_slab16", {gemm_skinny_kernel<OUT8, 4>, gemm_skinny_kernel<OUT32, 4>, gemm_skinny_kernel<OUT16, 4>}, 64, 16, 64, 512, true, true},  // 11
 };
+static const int SKINNY_CFG = 9;
 static const int g_num_configs = (int)(sizeof(g_configs) / sizeof(g_configs[0]));
 
 static int out_class(int out_dtype) {
@@ -658,6 +798,7 @@ static bool fast_eligible(const GemmParams& p) {
 // the LDS staging; the preferences were measured with weights streamed from HBM.
 static int pick_config(const GemmParams& p) {
   if (!fast_eligible(p)) return 0;
+  if (p.M <= 64) return SKINNY_CFG + (p.M > 16) + (p.M > 32);
   const bool wide_out = out_class(p.out_dtype) != OUT8;
   struct Cand { int cfg; double base; };
   const Cand cands[] = {
@@ -737,11 +878,25 @@ static int run(GemmParams p, int config, hipStream_t stream) {
   // the fast kernels quantise to int8 with round-half-even only; the truncating test switch runs
   // on the gather kernel
   const bool trunc8 = p.round_mode == TI_ROUND_TRUNC && out_class(p.out_dtype) == OUT8;
-  if (config < 0) config = trunc8 ? 0 : pick_config(p);
+  if (config < 0) config = (trunc8 && p.M > 64) ? 0 : pick_config(p);
   if (config >= g_num_configs) return fail(TI_E_COMBO, "config %d out of range", config);
   const Config& k = g_configs[config];
-  if (k.fast && trunc8) return fail(TI_E_COMBO, "config %s does not implement TI_ROUND_TRUNC for int8 outputs", k.name);
+  if (k.fast && !k.skinny && trunc8) return fail(TI_E_COMBO, "config %s does not implement TI_ROUND_TRUNC for int8 outputs", k.name);
   if (k.fast && !fast_eligible(p)) return fail(TI_E_COMBO, "config %s needs K-contiguous 16-byte aligned operands", k.name);
+  if (k.skinny) {
+    if (p.M > k.bm) return fail(TI_E_COMBO, "config %s needs M <= %d", k.name, k.bm);
+    // enough waves to fill the chip: split K between the waves of a workgroup when there are few slabs
+    const int64_t slabs = (int64_t)((p.N + 15) / 16) * p.batch;
+    const int ksteps = (p.K + 63) / 64;
+    int ksplit = 1;
+    while (ksplit < 8 && slabs * ksplit < 4096 && ksplit * 2 <= ksteps) ksplit *= 2;
+    p.ksplit = ksplit;
+    const int per_block = 8 / ksplit;
+    dim3 grid((unsigned)(((p.N + 15) / 16 + per_block - 1) / per_block), (unsigned)p.batch, 1);
+    g_last_config = config;
+    k.fn[out_class(p.out_dtype)]<<<grid, dim3(k.threads), 0, stream>>>(p);
+    return launch_status(k.name);
+  }
   p.tiles_m = (p.M + k.bm - 1) / k.bm;
   p.tiles_n = (p.N + k.bn - 1) / k.bn;
   if ((int64_t)p.tiles_m * p.tiles_n > 0x7fffffff) return fail(TI_E_SHAPE, "too many tiles");
@@ -769,7 +924,7 @@ int ti_bmm_i8_config(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk, con
   p.bias = bias; p.bias_kind = bias_kind;
   p.alpha = alpha; p.beta = beta;
   p.epilogue = epilogue; p.out_dtype = out_dtype; p.round_mode = round_mode;
-  p.tiles_m = p.tiles_n = 0; p.group_m = 1;
+  p.tiles_m = p.tiles_n = 0; p.group_m = 1; p.ksplit = 1;
   return ti::run(p, config, (hipStream_t)stream);
 }
 
