@@ -179,6 +179,19 @@ int ti_dq_add_layernorm_q(const int32_t* acc, int64_t acc_row_stride, float in_s
 int ti_gelu_q(const float* x, const float* scale, int8_t* y, int64_t n,
               int round_mode, void* stream);
 
+/*
+ * y_i8[r,j] = round_half_even( softmax_j(x_i8[r,:] * scale)[j] * 127 ), values in [0,127].
+ * The link between the two attention BMMs of a W8A8 decoder layer: int8 scores from
+ * bmm_s8t_s8n_s8t (kernels/bmm.py:576-612) in, int8 probabilities for the P.V BMM out.  The
+ * reference tree has no kernel for it (its modules stop at the BMMs); the arithmetic is the
+ * fp32 softmax followed by `mul(127).round()` that SmoothQuant-style callers of these modules do.
+ * scale is a host float (score scale).  causal_q_len > 0: rows come in groups of that many query
+ * positions, position i attends to columns 0 .. i + (cols - causal_q_len); 0 = no mask.
+ * cols <= 8192.  Row strides in elements, unit column stride.
+ */
+int ti_softmax_q(const int8_t* x, int64_t x_row_stride, float scale,
+                 int8_t* y, int64_t y_row_stride, int rows, int cols, int causal_q_len, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -45,7 +45,7 @@ def lib() -> ctypes.CDLL:
             build()
         _lib = ctypes.CDLL(_SO)
         for name in ("ti_oracle_bmm_i8", "ti_oracle_layernorm_q", "ti_oracle_dq_add_layernorm_q",
-                     "ti_oracle_gelu_q", "ti_oracle_gelu_f32"):
+                     "ti_oracle_gelu_q", "ti_oracle_gelu_f32", "ti_oracle_softmax_q"):
             getattr(_lib, name).restype = ctypes.c_int
     return _lib
 
@@ -207,3 +207,14 @@ def gelu_f32(x, scale):
     rc = lib().ti_oracle_gelu_f32(_p(x1), ps, _p(y), ctypes.c_int64(x1.size))
     assert rc == 0
     return y.reshape(x.shape)
+
+
+def softmax_q(x_i8, scale, causal_q_len=0):
+    """int8 scores [..., cols] -> int8 probabilities round(softmax(x*scale)*127)."""
+    x2 = np.ascontiguousarray(x_i8, dtype=np.int8).reshape(-1, x_i8.shape[-1])
+    rows, cols = x2.shape
+    y = np.empty((rows, cols), np.int8)
+    i64 = ctypes.c_int64
+    rc = lib().ti_oracle_softmax_q(_p(x2), i64(cols), ctypes.c_float(scale), _p(y), i64(cols), rows, cols, int(causal_q_len))
+    assert rc == 0
+    return y.reshape(x_i8.shape)

@@ -24,6 +24,8 @@
  *       == s*x exactly where representable.
  *   ti_oracle_gelu_q            kernels/fused.py:13,76-79
  *       pins: F.gelu(approximate="tanh"); gelu(0)=0; gelu(x)-gelu(-x)=x; saturation.
+ *   ti_oracle_softmax_q         (no reference function: the caller-side step between the two BMMs)
+ *       pins: torch.softmax(x*scale).mul(127).round(); rows sum to ~127; one-hot and uniform rows.
  *
  * Rounding contract: q8 = clamp(round_half_even(v), -128, 127), NaN -> 0 (mode 0); mode 1 is
  * the literal Triton `.to(int8)` truncation toward zero, clamped, kept as a test-time switch.
@@ -260,6 +262,35 @@ int ti_oracle_gelu_q(const float* x, const float* scale, int8_t* y, int64_t n, i
   const float s = *scale;
 #pragma omp parallel for schedule(static)
   for (int64_t i = 0; i < n; ++i) y[i] = q8(gelu_tanh_scaled(x[i], s), round_mode);
+  return 0;
+}
+
+/* int8 scores -> int8 probabilities: fp32 softmax of x*scale over the row (max-subtracted, libm expf,
+ * division per element), then round_half_even(p * 127) — `softmax(...).mul(127).round()` as
+ * SmoothQuant-style callers of the BMM modules do between bmm_s8t_s8n_s8t (kernels/bmm.py:576-612)
+ * and the P.V BMM; the reference tree itself has no such function, so there is nothing of the
+ * reference's to follow line by line.  Pins: torch.softmax on x*scale, mul(127), round
+ * (tests/test_oracle_rowops.py).  causal_q_len as in the HIP entry point. */
+int ti_oracle_softmax_q(const int8_t* x, int64_t x_row_stride, float scale, int8_t* y, int64_t y_row_stride,
+                        int rows, int cols, int causal_q_len) {
+#pragma omp parallel for schedule(static)
+  for (int r = 0; r < rows; ++r) {
+    const int8_t* xr = x + (int64_t)r * x_row_stride;
+    int8_t* yr = y + (int64_t)r * y_row_stride;
+    int limit = cols;
+    if (causal_q_len > 0) {
+      limit = (r % causal_q_len) + (cols - causal_q_len) + 1;
+      if (limit > cols) limit = cols;
+    }
+    int mx = -128;
+    for (int j = 0; j < limit; ++j) if (xr[j] > mx) mx = xr[j];
+    float sum = 0.0f;
+    for (int j = 0; j < limit; ++j) sum += expf((float)(xr[j] - mx) * scale);
+    for (int j = 0; j < cols; ++j) {
+      float p = j < limit ? expf((float)(xr[j] - mx) * scale) / sum : 0.0f;
+      yr[j] = q8(p * 127.0f, 0);
+    }
+  }
   return 0;
 }
 

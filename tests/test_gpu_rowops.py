@@ -152,3 +152,19 @@ def test_gelu_q_grid_and_module():
     want = O.gelu_q(x, np.float32(20.0))
     mx, rate = mismatch_report(got, want)
     assert mx <= 1 and rate < 1e-3
+
+
+@pytest.mark.parametrize("rows,cols,q_len", [(64, 2048, 0), (48, 2048, 16), (10, 300, 5), (7, 17, 0), (6, 4096, 3), (4, 8192, 0), (5, 1, 0)])
+def test_softmax_q(rows, cols, q_len):
+    fused = _fused()
+    g = rng(rows + cols)
+    x = g.integers(-128, 128, size=(rows, cols), dtype=np.int8)
+    for scale in (0.05, 0.5):
+        got = cpu(fused.softmax_q(gpu(x), scale, causal_q_len=q_len))
+        want = O.softmax_q(x, scale, causal_q_len=q_len)
+        mx, rate = mismatch_report(got, want)
+        print(f"softmax_q [{rows},{cols}] q_len {q_len} scale {scale}: max diff {mx}, mismatch rate {rate:.2e}")
+        assert mx <= 1 and rate <= max(2e-3, 1.5 / want.size)
+        assert got.min() >= 0
+    x3 = x.reshape(1, rows, cols)
+    assert fused.softmax_q(gpu(x3), 0.05).shape == (1, rows, cols)

@@ -138,3 +138,30 @@ def test_gelu_q_vs_torch_and_closed_forms():
     # saturation of the quantiser
     assert O.gelu_q(np.array([100.0], np.float32), scale)[0] == 127
     assert O.gelu_q(np.array([-0.75], np.float32), np.float32(1000.0))[0] == -128
+
+
+def test_softmax_q_vs_torch_softmax():
+    g = rng(21)
+    x = g.integers(-128, 128, size=(37, 300), dtype=np.int8)
+    x[0] = 5                      # uniform row
+    x[1] = -128; x[1, 17] = 127   # (nearly) one-hot row
+    for scale in (0.05, 0.5, 1e-3):
+        got = O.softmax_q(x, scale)
+        p = torch.softmax(torch.from_numpy(x).float() * scale, dim=-1)
+        want = p.mul(127).round().to(torch.int8).numpy()
+        diff = np.abs(got.astype(int) - want.astype(int))
+        assert diff.max() <= 1 and (diff != 0).mean() < 2e-3
+        frac = np.abs(p.numpy() * 127 - np.floor(p.numpy() * 127) - 0.5)
+        assert np.all(frac[diff != 0] < 1e-3)          # only rounding boundaries may differ
+        assert got.min() >= 0 and got.max() <= 127
+    assert np.all(O.softmax_q(x, 0.05)[0] == round(127 / 300))          # uniform row: 127/300 -> 0
+    oh = O.softmax_q(x, 0.5)[1]
+    assert oh[17] == 127 and oh.sum() == 127
+    # causal mask: position i of each group of q rows sees columns 0 .. i + (cols - q)
+    q_len, cols = 5, 12
+    xs = g.integers(-128, 128, size=(2 * q_len, cols), dtype=np.int8)
+    got = O.softmax_q(xs, 0.1, causal_q_len=q_len)
+    for r in range(2 * q_len):
+        lim = (r % q_len) + (cols - q_len) + 1
+        p = torch.softmax(torch.from_numpy(xs[r, :lim]).float() * 0.1, dim=-1).mul(127).round().numpy()
+        assert np.abs(got[r, :lim] - p).max() <= 1 and np.all(got[r, lim:] == 0)

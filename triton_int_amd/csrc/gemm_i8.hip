@@ -603,7 +603,7 @@ __global__ __launch_bounds__(256) void gemm_gather_kernel(GemmParams p) {
 // of A (the 16 x 16 result block has rows = n, columns = m).  Operands go from global memory
 // straight into registers in MFMA layout (lane = row + 16 * chunk); A is tiny and stays in L2.
 // The 8 waves of a workgroup either take 8 different slabs (short K) or split K between them
-// (k-steps interleaved, so that together they read consecutive bytes of a row) and add their
+// (each a contiguous run of k-steps, so a wave reads whole cache lines) and add their
 // int32 partial sums through LDS — integer addition, so the result does not depend on the split.
 template <int OUTCLS, int MBMAX>
 __global__ __launch_bounds__(512) void gemm_skinny_kernel(GemmParams p) {
@@ -632,19 +632,21 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(GemmParams p) {
 #pragma unroll
   for (int mb = 0; mb < MBMAX; ++mb) acc[mb] = (v4i){0, 0, 0, 0};
 
-  // This wave's k-steps are kpart, kpart + ksplit, ...  Whole 64-byte k-steps run in batches of U
+  // Whole 64-byte k-steps of this wave's run go in batches of U
   // with two register sets: the loads of batch b+1 are issued before the MFMAs of batch b, so a
   // wave keeps up to 2*U weight loads (1 KB each) in flight, and nothing in the batch loop looks
   // at a loaded value before the MFMAs do.  Left-over k-steps and a K tail (K % 64 != 0, the only
   // place that needs zero fill) are handled one at a time afterwards.  The weight stream bypasses
   // the caches (non-temporal); A is re-read by every slab and is served by L2.
   const int KSF = p.K >> 6;  // whole k-steps
-  const int nj = kpart < KSF ? (KSF - kpart + ksplit - 1) / ksplit : 0;
+  const int per = (KSF + ksplit - 1) / ksplit;  // each wave takes a contiguous run of k-steps
+  const int j0 = kpart * per;
+  const int nj = min(max(KSF - j0, 0), per);
   const int nb = nj / U;
-  const int kstride = ksplit * 64;
+  constexpr int kstride = 64;
   v4i wf[2][U], xf[2][U][MBMAX];
   auto load_batch = [&](int buf, int b) {
-    const int k0 = (kpart + b * U * ksplit) * 64;
+    const int k0 = (j0 + b * U) * 64;
 #pragma unroll
     for (int u = 0; u < U; ++u) wf[buf][u] = *(const v4i*)(wrow + k0 + u * kstride);
 #pragma unroll
@@ -670,7 +672,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(GemmParams p) {
   // left-over whole k-steps (fewer than U): one more batch, loads first, guarded by wave-uniform tests
   const int rem = nj - nb * U;
   if (rem > 0) {
-    const int k0 = (kpart + nb * U * ksplit) * 64;
+    const int k0 = (j0 + nb * U) * 64;
 #pragma unroll
     for (int u = 0; u < U - 1; ++u)
       if (u < rem) wf[0][u] = *(const v4i*)(wrow + k0 + u * kstride);
@@ -688,7 +690,7 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(GemmParams p) {
           acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[0][u], xf[0][u][mb], acc[mb], 0, 0, 0);
       }
   }
-  if ((p.K & 63) && kpart == KSF % ksplit) {
+  if ((p.K & 63) && kpart == 0) {
     const int k0 = KSF * 64;
     const bool ok = k0 + c4 * 16 < p.K;  // K is a multiple of 16: a chunk is all in or all out
     v4i w1 = *(const v4i*)(wrow + (ok ? k0 : 0));

@@ -217,6 +217,83 @@ static int launch_rownorm(const RowNormParams& p, hipStream_t stream) {
   return launch_status("rownorm_vec_kernel");
 }
 
+// ---- softmax -> int8 probabilities -------------------------------------------------------------
+// y = round_half_even(softmax(x_int8 * scale) * 127), the step between the two attention BMMs of a
+// W8A8 decoder layer (int8 scores in, int8 probabilities in [0,127] out).  One wavefront per row:
+// a lane holds VPT x 16 consecutive int8 scores, the row maximum is exact (integers), the
+// exponentials are kept in registers, and max / sum are wave reductions — no LDS, no barrier.
+// With causal_q_len > 0 the rows form groups of that many query positions and position i sees
+// columns 0 .. i + (cols - causal_q_len); masked columns get probability 0.
+constexpr int SM_WAVES = 4;
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+template <int VPT>
+__global__ __launch_bounds__(SM_WAVES * 64) void softmax_q_kernel(const int8_t* __restrict__ x, int64_t x_rs,
+                                                                  float scale, int8_t* __restrict__ y, int64_t y_rs,
+                                                                  int rows, int cols, int causal_q_len) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * SM_WAVES + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int limit = causal_q_len > 0 ? min(cols, (row % causal_q_len) + (cols - causal_q_len) + 1) : cols;
+  const int8_t* xr = x + (int64_t)row * x_rs;
+  int8_t* yr = y + (int64_t)row * y_rs;
+  const bool vec = ((((uintptr_t)xr) | ((uintptr_t)yr)) & 15) == 0;
+
+  int v[VPT][16];
+  int mx = -128;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int c0 = (j * 64 + lane) * 16;
+    if (vec && c0 + 16 <= cols) {
+      const v4i w = __builtin_nontemporal_load((const v4i*)(xr + c0));
+#pragma unroll
+      for (int t = 0; t < 16; ++t) v[j][t] = (int)(int8_t)(w[t >> 2] >> ((t & 3) * 8));
+    } else {
+#pragma unroll
+      for (int t = 0; t < 16; ++t) v[j][t] = c0 + t < cols ? (int)xr[c0 + t] : -128;
+    }
+#pragma unroll
+    for (int t = 0; t < 16; ++t)
+      if (c0 + t < limit) mx = max(mx, v[j][t]);
+  }
+  mx = (int)wave_max((float)mx);  // |x| <= 128: exact in fp32
+  float e[VPT][16];
+  float sum = 0.0f;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int c0 = (j * 64 + lane) * 16;
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+      const float ex = __expf((float)(v[j][t] - mx) * scale);
+      e[j][t] = c0 + t < limit ? ex : 0.0f;
+      sum += e[j][t];
+    }
+  }
+  sum = wave_sum(sum);
+  const float r = 127.0f / sum;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int c0 = (j * 64 + lane) * 16;
+    unsigned w[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+      w[g] = pack4(q8<false>(e[j][4 * g] * r), q8<false>(e[j][4 * g + 1] * r), q8<false>(e[j][4 * g + 2] * r),
+                   q8<false>(e[j][4 * g + 3] * r));
+    if (vec && c0 + 16 <= cols) {
+      __builtin_nontemporal_store((v4u){w[0], w[1], w[2], w[3]}, (v4u*)(yr + c0));
+    } else {
+#pragma unroll
+      for (int t = 0; t < 16; ++t)
+        if (c0 + t < cols) yr[c0 + t] = (int8_t)(w[t >> 2] >> ((t & 3) * 8));
+    }
+  }
+}
+
 // ---- GELU -> int8 ---------------------------------------------------------------------------
 
 constexpr int GQ_THREADS = 256;
@@ -295,6 +372,26 @@ int ti_dq_add_layernorm_q(const int32_t* acc, int64_t acc_row_stride, float in_s
   p.rows = rows; p.cols = cols; p.rms = 0; p.round_mode = round_mode;
   p.mean_out = mean_out; p.rstd_out = rstd_out;
   return ti::launch_rownorm<true>(p, (hipStream_t)stream);
+}
+
+int ti_softmax_q(const int8_t* x, int64_t x_row_stride, float scale, int8_t* y, int64_t y_row_stride, int rows,
+                 int cols, int causal_q_len, void* stream) {
+  if (rows < 0 || cols < 0 || causal_q_len < 0) return ti::fail(TI_E_SHAPE, "negative size");
+  if (rows == 0 || cols == 0) return TI_OK;
+  if (!x || !y) return ti::fail(TI_E_NULL, "x and y are required");
+  if (causal_q_len > cols) return ti::fail(TI_E_SHAPE, "causal_q_len %d > cols %d", causal_q_len, cols);
+  if (causal_q_len > 0 && rows % causal_q_len) return ti::fail(TI_E_SHAPE, "rows %d not a multiple of causal_q_len %d", rows, causal_q_len);
+  if (cols > 64 * 16 * 8) return ti::fail(TI_E_SHAPE, "softmax rows longer than 8192 are not supported");
+  int rc = ti::check_device();
+  if (rc != TI_OK) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid((unsigned)((rows + ti::SM_WAVES - 1) / ti::SM_WAVES)), block(ti::SM_WAVES * 64);
+  const int vpt = (cols + 1023) / 1024;
+  if (vpt <= 1) ti::softmax_q_kernel<1><<<grid, block, 0, s>>>(x, x_row_stride, scale, y, y_row_stride, rows, cols, causal_q_len);
+  else if (vpt <= 2) ti::softmax_q_kernel<2><<<grid, block, 0, s>>>(x, x_row_stride, scale, y, y_row_stride, rows, cols, causal_q_len);
+  else if (vpt <= 4) ti::softmax_q_kernel<4><<<grid, block, 0, s>>>(x, x_row_stride, scale, y, y_row_stride, rows, cols, causal_q_len);
+  else ti::softmax_q_kernel<8><<<grid, block, 0, s>>>(x, x_row_stride, scale, y, y_row_stride, rows, cols, causal_q_len);
+  return ti::launch_status("softmax_q_kernel");
 }
 
 int ti_gelu_q(const float* x, const float* scale, int8_t* y, int64_t n, int round_mode, void* stream) {

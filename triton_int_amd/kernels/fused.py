@@ -103,3 +103,24 @@ def gelu_q(x, scale, *, _round_mode=L.ROUND_RNE_CLAMP):
         rc = L.lib().ti_gelu_q(L.ptr(x), L.ptr(s), L.ptr(y), x.numel(), int(_round_mode), L.current_stream(x.device))
     L.check(rc, "ti_gelu_q")
     return y
+
+
+def softmax_q(x, scale, causal_q_len=0):
+    """int8 attention scores [..., cols] -> int8 probabilities round(softmax(x * scale) * 127) in [0, 127].
+    The reference has no kernel for this step (callers of its BMM modules do it in fp32 torch between
+    bmm_s8t_s8n_s8t and the P.V BMM).  `scale` is a python float; causal_q_len > 0 masks position i of
+    every group of causal_q_len rows to columns 0 .. i + (cols - causal_q_len)."""
+    L.require_cuda(x)
+    assert x.dtype == torch.int8, "scores must be int8"
+    cols = x.shape[-1]
+    x2 = x.reshape(-1, cols)
+    if x2.stride(1) != 1:
+        x2 = x2.contiguous()
+    rows = x2.shape[0]
+    y = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    y2 = y.view(-1, cols)
+    with torch.cuda.device(x.device):
+        rc = L.lib().ti_softmax_q(L.ptr(x2), x2.stride(0) if rows > 1 else cols, float(scale), L.ptr(y2), cols, rows,
+                                  cols, int(causal_q_len), L.current_stream(x.device))
+    L.check(rc, "ti_softmax_q")
+    return y

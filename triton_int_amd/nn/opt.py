@@ -1,0 +1,114 @@
+"""A W8A8 OPT-shaped decoder layer assembled from the int8 modules.
+
+Not part of the reference tree: its modules are the building blocks ("For qkv_proj", "For fc1",
+"For fc2 and out_proj", nn/linear.py:19,71,126) and the layer that chains them lives in the
+caller (SmoothQuant-style Int8OPTDecoderLayer).  This module is that caller for benchmarks and
+end-to-end tests: every heavy step is one of the package's HIP kernels, torch only reshapes.
+
+    hidden fp32 [B,S,H]
+      LayerNormQ -> int8                                    (layer_norm_fwd_fused_single_pass_q)
+      q,k,v = W8A8B8O8Linear -> int8                        (linear_a8_w8_b8_o8)
+      scores = BMM_S8T_S8N_S8T(q, k) -> int8                (bmm_s8t_s8n_s8t)
+      probs  = softmax_q(scores, causal) -> int8 [0,127]    (ti_softmax_q)
+      ctx    = BMM_S8T_S8N_S8T(probs, v^T) -> int8, written head-merged through output strides
+      acc    = W8A8B32O32LinearWithoutScaling(ctx) -> int32 (linear_a8_w8_b32_o32)   out_proj
+      resid, h8 = DQ_Add_LayerNorm_Q(hidden, acc)           (ti_dq_add_layernorm_q)
+      f8     = W8A8BFP32OFP32_GeLu_Q(h8) -> int8            (GEMM + GELU-quant epilogue)   fc1
+      out    = W8A8BFP32OFP32Linear(f8) + resid -> fp32                                  fc2
+"""
+from __future__ import annotations
+
+import torch
+
+from ..kernels.bmm import bmm_s8t_s8n_s8t
+from ..kernels.fused import softmax_q
+from .fused import DQ_Add_LayerNorm_Q, LayerNormQ, W8A8BFP32OFP32_GeLu_Q
+from .linear import W8A8B8O8Linear, W8A8B32O32LinearWithoutScaling, W8A8BFP32OFP32Linear
+
+
+class W8A8OPTDecoderLayer(torch.nn.Module):
+    def __init__(self, hidden=5120, heads=40, ffn=20480, causal=True):
+        super().__init__()
+        assert hidden % heads == 0
+        self.hidden, self.heads, self.head_dim, self.ffn, self.causal = hidden, heads, hidden // heads, ffn, causal
+        self.ln1 = LayerNormQ(hidden)
+        self.q_proj = W8A8B8O8Linear(hidden, hidden)
+        self.k_proj = W8A8B8O8Linear(hidden, hidden)
+        self.v_proj = W8A8B8O8Linear(hidden, hidden)
+        self.out_proj = W8A8B32O32LinearWithoutScaling(hidden, hidden)
+        self.ln2 = DQ_Add_LayerNorm_Q(hidden)
+        self.fc1 = W8A8BFP32OFP32_GeLu_Q(hidden, ffn)
+        self.fc2 = W8A8BFP32OFP32Linear(ffn, hidden)
+        # attention scales: int8 scores = q8(qk_alpha * q.k), probabilities = softmax(scores * score_scale),
+        # int8 context = q8(pv_alpha * P.V)
+        self.qk_alpha = 1e-3
+        self.score_scale = 0.05
+        self.pv_alpha = 1.0 / 127.0
+
+    @torch.no_grad()
+    def randomize(self, seed=0):
+        """Random int8 weights and per-tensor scales drawn uniformly from [1e-3, 1e-2]."""
+        g = torch.Generator(device="cpu").manual_seed(seed)
+
+        def s():
+            return float(torch.empty(1).uniform_(1e-3, 1e-2, generator=g))
+
+        for lin in (self.q_proj, self.k_proj, self.v_proj, self.out_proj, self.fc1, self.fc2):
+            lin.weight = torch.randint(-127, 128, tuple(lin.weight.shape), dtype=torch.int8, generator=g).to(lin.weight.device)
+        for lin in (self.q_proj, self.k_proj, self.v_proj):
+            lin.bias = torch.randint(-127, 128, (self.hidden,), dtype=torch.int8, generator=g).to(lin.bias.device)
+            lin.a = torch.tensor(s() / 10, dtype=torch.float32, device=lin.a.device)
+            lin.b = torch.tensor(s(), dtype=torch.float32, device=lin.b.device)
+        self.out_proj.bias = torch.randint(-1000, 1000, (self.hidden,), dtype=torch.int32, generator=g).to(self.out_proj.bias.device)
+        self.ln2.input_scale = s() / 100
+        self.fc1.bias = torch.randn(self.ffn, generator=g).to(self.fc1.bias.device)
+        self.fc1.a = torch.tensor(s() / 30, dtype=torch.float32, device=self.fc1.a.device)
+        self.fc1.b = torch.tensor(20.0, dtype=torch.float32, device=self.fc1.b.device)
+        self.fc2.bias = torch.randn(self.hidden, generator=g).to(self.fc2.bias.device)
+        self.fc2.a = torch.tensor(s() / 100, dtype=torch.float32, device=self.fc2.a.device)
+        for ln in (self.ln1, self.ln2):
+            ln.weight = (torch.randn(self.hidden, generator=g) * 0.1 + 1.0).div(0.05).to(ln.weight.device)
+            ln.bias = (torch.randn(self.hidden, generator=g) * 0.1).div(0.05).to(ln.bias.device)
+        return self
+
+    def _heads(self, t, B, S):
+        # [B,S,H] int8 -> [B*heads, S, D] (a copy: the BMM wants each head's rows contiguous in K)
+        return t.view(B, S, self.heads, self.head_dim).transpose(1, 2).reshape(B * self.heads, S, self.head_dim)
+
+    @torch.no_grad()
+    def forward(self, hidden, kv_cache=None, _trace=None):
+        """hidden fp32 [B,S,H].  kv_cache = (K int8 [B*heads, T, D], V^T int8 [B*heads, D, T]) holds the
+        T-S earlier positions in its first T-S slots; the S new positions are written into the last S
+        slots before attention (decode / chunked prefill).  Returns fp32 [B,S,H].  A dict passed as
+        `_trace` receives every intermediate tensor (for stage-by-stage parity tests)."""
+        B, S, H = hidden.shape
+        h8 = self.ln1(hidden)
+        q = self._heads(self.q_proj(h8), B, S)
+        k_new = self._heads(self.k_proj(h8), B, S)
+        v_new = self._heads(self.v_proj(h8), B, S)
+        if kv_cache is None:
+            k_all, vt_all = k_new, v_new.transpose(1, 2).contiguous()
+        else:
+            k_all, vt_all = kv_cache
+            T = k_all.shape[1]
+            k_all[:, T - S:, :] = k_new
+            vt_all[:, :, T - S:] = v_new.transpose(1, 2)
+        T = k_all.shape[1]
+        scores = bmm_s8t_s8n_s8t(q, k_all, self.qk_alpha)                           # [B*heads, S, T] int8
+        probs = softmax_q(scores, self.score_scale, causal_q_len=S if self.causal else 0)
+        # P.V with the head merge folded into the output strides: head h of batch b writes columns
+        # h*D .. h*D+D of row (b, s) of a [B,S,H] tensor
+        ctx = torch.empty((B, S, H), dtype=torch.int8, device=hidden.device)
+        for b in range(B):
+            out_view = ctx[b].view(S, self.heads, self.head_dim).transpose(0, 1)   # [heads, S, D] strided
+            bmm_s8t_s8n_s8t(probs[b * self.heads:(b + 1) * self.heads], vt_all[b * self.heads:(b + 1) * self.heads],
+                            self.pv_alpha, out=out_view)
+        acc = self.out_proj(ctx)                                                    # int32 [B,S,H]
+        resid, h8b = self.ln2(hidden, acc)
+        f8 = self.fc1(h8b)
+        y = self.fc2(f8)
+        out = y + resid
+        if _trace is not None:
+            _trace.update(h8=h8, q=q, k_all=k_all, vt_all=vt_all, scores=scores, probs=probs, ctx=ctx, acc=acc,
+                          resid=resid, h8b=h8b, f8=f8, fc2=y, out=out)
+        return out
