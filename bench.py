@@ -158,8 +158,51 @@ def extras(torch, dev):
     of = torch.empty((B, S, D), dtype=torch.float32, device=dev)
     ms = time_region(torch, lambda: bmm.bmm_s8t_s8n_f32t(p, vt, 1.0 / 16129, out=of), 10, 2)
     out["bmm_pv_f32_160x2048x128x2048"] = {"ms": ms, "GBps": 880.8e6 / ms / 1e6, "TOPS": 171.8e9 / ms / 1e9}
+    del q, k, sc, vt, of
+    # int8 scores -> int8 probabilities (softmax + quantise), 2 B/element
+    ms = time_region(torch, lambda: fused.softmax_q(p, 0.05), 10, 2)
+    out["softmax_q_160x2048x2048"] = {"ms": ms, "GBps": p.numel() * 2 / ms / 1e6}
+    del p
     for v in out.values():
         v["frac_hbm_peak"] = v["GBps"] / HBM_PEAK_GBPS
+    return out
+
+
+def decoder_layer_ms(torch, dev):
+    """W8A8 OPT-13B-shaped decoder layer (hidden 5120, 40 heads, FFN 20480), random int8 weights:
+    prefill (batch 1, seq 2048) and decode (16 tokens against a 2048-long int8 KV).  Two layers with
+    different weights alternate so that no weight is cache-resident."""
+    from triton_int_amd.nn.opt import W8A8OPTDecoderLayer
+
+    layers = [W8A8OPTDecoderLayer().randomize(seed=i).to(dev) for i in range(2)]
+    x = torch.randn((1, 2048, 5120), device=dev)
+    state = {"i": 0}
+
+    def prefill():
+        state["i"] ^= 1
+        layers[state["i"]](x)
+
+    out = {"prefill_1x2048_ms": time_region(torch, prefill, 10, 2)}
+    kc = torch.randint(-127, 128, (40, 2048, 128), dtype=torch.int8, device=dev)
+    vc = torch.randint(-127, 128, (40, 128, 2048), dtype=torch.int8, device=dev)
+    xd = torch.randn((1, 16, 5120), device=dev)
+
+    def decode():
+        state["i"] ^= 1
+        layers[state["i"]](xd, kv_cache=(kc, vc))
+
+    out["decode_16tok_kv2048_eager_ms"] = time_region(torch, decode, 20, 3)
+    # the same two layers replayed from a HIP graph: launch overhead removed
+    graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        decode(); decode()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            decode(); decode()
+    torch.cuda.synchronize()
+    out["decode_16tok_kv2048_graph_ms"] = time_region(torch, graph.replay, 10, 2) / 2
+    out["gemm_bmm_ops_prefill"] = 1374.4e9
+    out["prefill_tops"] = 1374.4e9 / (out["prefill_1x2048_ms"] * 1e-3) / 1e12
     return out
 
 
@@ -263,6 +306,7 @@ def main():
     result["roofline"]["frac_of_measured_issue_peak"] = achieved / peak_rand
     if not args.no_extra:
         result["extra"] = extras(torch, dev)
+        result["extra"]["opt13b_decoder_layer"] = decoder_layer_ms(torch, dev)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch, layers)
     print(json.dumps(result))

@@ -16,13 +16,19 @@ def _lib():
     return L
 
 
-def _configs(M=1):
-    """(index, name) of every kernel configuration that can run M activation rows"""
+def _configs(M=1, N=None, out8=False):
+    """(index, name) of every kernel configuration that can run M activation rows (and, for the
+    persistent "stream" kernels with an int8 output, N output columns: they store whole 16-byte
+    segments of a row)"""
     L = _lib()
     n = L.lib().ti_gemm_num_configs()
     out = [(i, L.lib().ti_gemm_config_name(i).decode()) for i in range(n)]
     def fits(nm):  # "skinny_m<rows>_..." configurations take at most <rows> activation rows
-        return not nm.startswith("skinny") or M <= int(nm.split("_")[1][1:])
+        if nm.startswith("skinny"):
+            return M <= int(nm.split("_")[1][1:])
+        if nm.startswith("stream") and out8:
+            return N is not None and N % 16 == 0
+        return True
     return [(i, nm) for i, nm in out if fits(nm)]
 
 
@@ -63,7 +69,7 @@ def test_all_configs_int8_epilogues_bit_exact(shape):
         want = O.linear_a8_w8_b8_o8(a, w, bias, alpha, beta)
         want_relu = O.linear_relu_a8_w8_b8_o8(a, w, bias, alpha, beta)
         want_tr = O.linear_a8_w8_b8_o8(a, w, bias, alpha, beta, round_mode=O.TRUNC)
-        for cfg, name in _configs(M):
+        for cfg, name in _configs(M, N, out8=True):
             got = cpu(linear.linear_a8_w8_b8_o8(ga, gw, gb, alpha, beta, _config=cfg))
             assert np.array_equal(got, want), f"o8 config {name} alpha {alpha}"
             got = cpu(linear.linear_relu_a8_w8_b8_o8(ga, gw, gb, alpha, beta, _config=cfg))
@@ -114,7 +120,7 @@ def test_all_configs_gelu_q(shape):
     want = O.linear_a8_w8_bfp32_ofp32_GeLu_Q(a, w, bias, alpha, beta)
     assert np.unique(want).size > 100  # the case really exercises the rounding, not only the clamp
     ga, gw, gb = gpu(a), gpu(w), gpu(bias)
-    for cfg, name in _configs(M):
+    for cfg, name in _configs(M, N, out8=True):
         got = cpu(fused.linear_a8_w8_bfp32_ofp32_GeLu_Q(ga, gw, gb, alpha, beta, _config=cfg))
         mx, rate = mismatch_report(got, want)
         assert mx <= 1 and rate < 1e-3, f"{name}: max {mx} rate {rate}"
@@ -170,10 +176,37 @@ def test_bmm_fast_path_all_configs(B, M, N, K):
     alpha = np.float32(1e-3)
     want8 = O.bmm_s8t_s8n_s8t(a, b, alpha)
     wantf = O.bmm_s8t_s8n_f32t(a, b, alpha)
+    out8_ok = {c for c, _ in _configs(M, N, out8=True)}
     for cfg, name in _configs(M):
+        assert np.array_equal(cpu(bmm.bmm_s8t_s8n_s32t(ga, gb, _config=cfg)), want32), name
+        if cfg in out8_ok:
+            assert np.array_equal(cpu(bmm.bmm_s8t_s8n_s8t(ga, gb, alpha, _config=cfg)), want8), name
+        assert np.array_equal(cpu(bmm.bmm_s8t_s8n_f32t(ga, gb, alpha, _config=cfg)), wantf), name
+
+
+# The persistent kernels walk several tiles per workgroup with the operand loads of the next tile
+# in flight during the epilogue of the current one: these shapes give every workgroup more than
+# one tile (more than 768 tiles of 128x128, more than 256 of 256x256), ragged in M, N and K, with
+# one, two and many k-tiles per tile.
+@pytest.mark.parametrize("B,M,N,K", [(80, 500, 464, 48), (80, 500, 464, 128), (72, 520, 496, 400), (1, 4100, 4368, 208)])
+def test_stream_configs_many_tiles_per_workgroup(B, M, N, K):
+    _, bmm, _ = _kl()
+    g = rng(B + M + K)
+    a, b = rand_i8(g, B, M, K), rand_i8(g, B, N, K)
+    ga, gb = gpu(a), gpu(b)
+    want32 = O.bmm_s8t_s8n_s32t(a, b)
+    alpha = np.float32(2.5 / (np.sqrt(K) * 127 * 127 / 3))
+    want8 = O.bmm_s8t_s8n_s8t(a, b, alpha)
+    wantf = O.bmm_s8t_s8n_f32t(a, b, alpha)
+    ran = 0
+    for cfg, name in _configs(M, N, out8=True):
+        if not name.startswith("stream"):
+            continue
+        ran += 1
         assert np.array_equal(cpu(bmm.bmm_s8t_s8n_s32t(ga, gb, _config=cfg)), want32), name
         assert np.array_equal(cpu(bmm.bmm_s8t_s8n_s8t(ga, gb, alpha, _config=cfg)), want8), name
         assert np.array_equal(cpu(bmm.bmm_s8t_s8n_f32t(ga, gb, alpha, _config=cfg)), wantf), name
+    assert ran >= 1
 
 
 def test_odd_k_and_unaligned_fall_back_to_gather():

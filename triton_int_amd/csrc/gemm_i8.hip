@@ -44,11 +44,7 @@ __device__ unsigned long long ti_trace_buf[8192];
 // block ids are first folded into 8 contiguous ranges (one per XCD) and each range then walks
 // the tile grid in column-major groups of `group_m` row-tiles so that a range re-uses few
 // distinct A and B panels.
-__device__ __forceinline__ void tile_coords(const GemmParams& p, int pid, int& tm, int& tn) {
-  const int T = p.tiles_m * p.tiles_n;
-  const int xcd = pid & 7, local = pid >> 3;
-  const int per = T >> 3, rem = T & 7;
-  const int lid = xcd * per + min(xcd, rem) + local;
+__device__ __forceinline__ void tile_from_rank(const GemmParams& p, int lid, int& tm, int& tn) {
   const int gsz = p.group_m * p.tiles_n;
   const int gid = lid / gsz;
   const int first_m = gid * p.group_m;
@@ -56,6 +52,28 @@ __device__ __forceinline__ void tile_coords(const GemmParams& p, int pid, int& t
   const int r = lid - gid * gsz;
   tm = first_m + r % gm;
   tn = r / gm;
+}
+
+__device__ __forceinline__ void tile_coords(const GemmParams& p, int pid, int& tm, int& tn) {
+  const int T = p.tiles_m * p.tiles_n;
+  const int xcd = pid & 7, local = pid >> 3;
+  const int per = T >> 3, rem = T & 7;
+  tile_from_rank(p, xcd * per + min(xcd, rem) + local, tm, tn);
+}
+
+// Batched launches (grid = tiles x batch): the same folding applied to the whole tiles*batch
+// sequence, so that one XCD works through whole batches and its L2 fetches every operand panel of
+// a batch once instead of all 8 L2s fetching most of every batch.
+__device__ __forceinline__ void batch_tile_coords(const GemmParams& p, int pid, int by, int nbatch, int& bz, int& tm,
+                                                  int& tn) {
+  const int T = p.tiles_m * p.tiles_n;
+  const int W = T * nbatch;
+  const int lin = by * T + pid;
+  const int xcd = lin & 7, local = lin >> 3;
+  const int per = W >> 3, rem = W & 7;
+  const int g = xcd * per + min(xcd, rem) + local;
+  bz = g / T;
+  tile_from_rank(p, g - bz * T, tm, tn);
 }
 
 // ---- epilogue (shared by both kernel families) ------------------------------------------------
@@ -205,8 +223,10 @@ __device__ __forceinline__ void wait_loads_and_barrier() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
 }
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int SWZ, int NSTAGE, int OUTCLS>
-__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmParams p) {
+// OCC = workgroups the register allocation must allow per CU (short-K batched shapes want two or
+// three co-resident workgroups so that one's epilogue overlaps another's loads).
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int SWZ, int NSTAGE, int OUTCLS, int OCC = 1>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3) / 4) void gemm_mfma_kernel(GemmParams p) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int CH = BK / 16;
   constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
@@ -214,26 +234,26 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmPa
   constexpr int KS = BK / 32;  // MFMA k-steps per k-tile
   constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
   constexpr int STAGE = A_BYTES + B_BYTES;
-  constexpr int C_PITCH = BN + 4;  // int8 staging pitch: 33-dword rows keep dword writes conflict-free
-  constexpr int LDS_BYTES = (NSTAGE * STAGE > BM * C_PITCH) ? NSTAGE * STAGE : BM * C_PITCH;
+  constexpr int LDS_BYTES = NSTAGE * STAGE;
   constexpr int DEPTH = NSTAGE - 1;  // k-tiles of loads in flight
   static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % 64 == 0, "tile shape");
   static_assert(NSTAGE >= 3 && LDS_BYTES <= 160 * 1024, "LDS budget");
 
   __shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];
-#ifdef TI_TRACE
-  const uint64_t tr_entry = wall_clock64();
-#endif
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
-  int tile_m, tile_n;
-  tile_coords(p, blockIdx.x, tile_m, tile_n);
+  int tile_m, tile_n, bz = 0;
+  if (gridDim.y == 1) tile_coords(p, blockIdx.x, tile_m, tile_n);
+  else batch_tile_coords(p, blockIdx.x, blockIdx.y, gridDim.y, bz, tile_m, tile_n);
+  // the divisions above run on the vector unit; the results are uniform and feed scalar operands
+  bz = __builtin_amdgcn_readfirstlane(bz);
+  tile_m = __builtin_amdgcn_readfirstlane(tile_m);
+  tile_n = __builtin_amdgcn_readfirstlane(tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
-  const int bz = blockIdx.y;
 
   const int8_t* Ab = p.A + (int64_t)bz * p.sAb;
   const int8_t* Bb = p.B + (int64_t)bz * p.sBb;
@@ -264,9 +284,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmPa
   // flight, and so the vmcnt to wait for, constant.
   int k_issue = 0, st_issue = 0;
   auto dma = [&](int d) {
-#if defined(TI_ABLATE) && TI_ABLATE == 1
-    return;  // debug build: no global loads
-#endif
     if (d < A_IT) {
       const unsigned dst = wave_slot + st_issue * STAGE + d * NT * 16;
       dma16_to_lds(rA, (k_issue < la.klim[d]) ? la.voff[d] : OOB, k_issue, dst);
@@ -306,10 +323,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmPa
   };
   auto mfma = [&](int buf, int u) {
     const int i = u / TN, j = u % TN;
-#if defined(TI_ABLATE) && TI_ABLATE == 2
-    acc[i][j][0] += fa[buf][i][0] ^ fb[buf][j][0];  // debug build: no MFMA, keep the operands live
-    return;
-#endif
     if constexpr (OUTCLS == OUT8)  // rows of the MFMA result = n (4 consecutive n per lane)
       acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
     else  // rows of the MFMA result = m, lanes run along n
@@ -357,9 +370,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmPa
     for (int r = 0; r < NR; ++r) load_frag(lds, 0, 0, r);
   }
 
-#ifdef TI_TRACE
-  uint64_t tr_wait = 0, tr_bar = 0, tr_t0 = __builtin_readcyclecounter(), tr_w0 = wall_clock64();
-#endif
   int st = 0;
   for (int kt = 0; kt < KT; ++kt) {
     const char* cur = lds + st * STAGE;
@@ -374,34 +384,15 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmPa
     // every LDS read of this k-tile is issued.  Wait for them and for k-tile kt+1 to have landed
     // (younger loads may stay in flight), then let the workgroup agree: after the barrier the
     // stage of k-tile kt+1 is readable and this k-tile's stage may be overwritten.
-#ifdef TI_TRACE
-    const uint64_t tr_a = __builtin_readcyclecounter();
-    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LOADS*(DEPTH - 2) + LOADS_A) : "memory");
-    const uint64_t tr_b = __builtin_readcyclecounter();
-    asm volatile("s_barrier" ::: "memory");
-    const uint64_t tr_c = __builtin_readcyclecounter();
-    tr_wait += tr_b - tr_a;
-    tr_bar += tr_c - tr_b;
-#else
     wait_loads_and_barrier<LOADS*(DEPTH - 2) + LOADS_A>();
-#endif
     // last k-step: first fragments of the next k-tile, part B of the fetch
     kstep((KS - 1) & 1, lds + st * STAGE, 0, kt + 1 < KT, LOADS_A, LOADS_B);
     dma_advance();
   }
-#ifdef TI_TRACE
-  const uint64_t tr_t1 = __builtin_readcyclecounter(), tr_w1 = wall_clock64();
-#endif
   // the trailing (out-of-bounds) loads still write zeros into LDS: drain before re-using it
   wait_loads_and_barrier<0>();
 
   // ---- epilogue ----
-#ifdef TI_TRACE
-  if (lane == 0 && blockIdx.x < 256) {
-    unsigned long long* t = ti_trace_buf + (blockIdx.x * 4 + wave) * 8;
-    t[0] = tr_t1 - tr_t0; t[1] = tr_wait; t[2] = tr_bar; t[3] = tr_entry; t[4] = tr_w0; t[5] = tr_w1 - tr_w0;
-  }
-#endif
   // The per-element code below is fully unrolled over the accumulator registers, so everything
   // that depends on the epilogue kind is decided once, outside the unrolled part: one uniform
   // branch selects a specialised body, and the remaining run-time options (rounding mode, ReLU,
@@ -413,14 +404,18 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmPa
 
   if constexpr (OUTCLS == OUT8) {
     // acc[i][j][r]: m = m0 + wm*WTM + i*32 + lrow;  n = n0 + wn*WTN + j*32 + 8*(r/4) + 4*lhi + r%4.
-    // Quantise, pack 4 consecutive n into a dword, stage the tile in LDS, then write rows with
-    // 16-byte stores.  (The K loop ended with a barrier, so the operand stages are free.)
+    // Quantise and pack 4 consecutive n into a dword X[g] (g = r/4).  Lanes l and l+32 hold the two
+    // halves of every 8-byte group of a row, so two half-wave swaps, (X0, X2) and (X1, X3), leave
+    // lane l with bytes 0..15 and lane l+32 with bytes 16..31 of the row's 32-byte segment: one
+    // 16-byte store per 32x32 block and lane, no trip through LDS.
     // Per element: cvt, mul, (add), clamp in fp32 (v_med3_f32), then one add of 1.5*2^23: that
     // add rounds to the nearest integer, ties to even, and leaves the two's-complement int8 in the
     // low byte of the float's bit pattern.  Clamping first keeps the sum in the exact range; since
     // the bounds are integers, clamp-then-round equals round-then-clamp.  ReLU is a lower bound of 0.
     // (Truncation, the test-time rounding switch, is served by the gather kernel instead.)
     const float q_floor = e.epilogue == TI_EPI_SCALE_RELU_I8 ? 0.0f : -128.0f;
+    int8_t* Cz = (int8_t*)Cb + (int64_t)bz * p.sCb;
+    const bool vec_ok = ((p.sCm & 15) == 0) && ((((uintptr_t)Cz) & 15) == 0);
     auto body = [&](auto gelu_tag, auto bias_tag) {
       constexpr bool GELU = decltype(gelu_tag)::value;
       constexpr bool BIAS = decltype(bias_tag)::value;
@@ -433,24 +428,40 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmPa
       };
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
+        const int nj = n0 + wn * WTN + j * 32;
+        float col[4][4];
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int nl = wn * WTN + j * 32 + 8 * g + 4 * lhi;
-          float col[4] = {0.f, 0.f, 0.f, 0.f};
-          if constexpr (BIAS) {
+        for (int g = 0; g < 4; ++g)
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
-              col[t] = column_term_t<GELU ? TI_BIAS_F32 : TI_BIAS_I8>(e, min(n0 + nl + t, p.N - 1), GELU);
+          for (int t = 0; t < 4; ++t) {
+            if constexpr (BIAS)
+              col[g][t] = column_term_t<GELU ? TI_BIAS_F32 : TI_BIAS_I8>(e, min(nj + 8 * g + 4 * lhi + t, p.N - 1), GELU);
+            else
+              col[g][t] = 0.0f;
           }
+        const int n = nj + 16 * lhi;
 #pragma unroll
-          for (int i = 0; i < TM; ++i) {
-            const int ml = wm * WTM + i * 32 + lrow;
-            const unsigned b0 = one(acc[i][j][4 * g + 0], col[0]), b1 = one(acc[i][j][4 * g + 1], col[1]);
-            const unsigned b2 = one(acc[i][j][4 * g + 2], col[2]), b3 = one(acc[i][j][4 * g + 3], col[3]);
+        for (int i = 0; i < TM; ++i) {
+          unsigned X[4];
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const unsigned b0 = one(acc[i][j][4 * g + 0], col[g][0]), b1 = one(acc[i][j][4 * g + 1], col[g][1]);
+            const unsigned b2 = one(acc[i][j][4 * g + 2], col[g][2]), b3 = one(acc[i][j][4 * g + 3], col[g][3]);
             // low bytes of b0..b3 -> one dword
-            const unsigned lo = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u);
-            const unsigned hi = __builtin_amdgcn_perm(b3, b2, 0x04000c0cu);
-            *(unsigned*)(lds + ml * C_PITCH + nl) = lo | hi;
+            X[g] = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u) | __builtin_amdgcn_perm(b3, b2, 0x04000c0cu);
+          }
+          const auto s02 = __builtin_amdgcn_permlane32_swap(X[0], X[2], false, false);
+          const auto s13 = __builtin_amdgcn_permlane32_swap(X[1], X[3], false, false);
+          v4u v;
+          v[0] = s02[0]; v[1] = s02[1]; v[2] = s13[0]; v[3] = s13[1];
+          const int m = m0 + wm * WTM + i * 32 + lrow;
+          if (m >= p.M || n >= p.N) continue;
+          int8_t* dst = Cz + (int64_t)m * p.sCm + n;
+          if (vec_ok && n + 16 <= p.N) {
+            *(v4u*)dst = v;
+          } else {
+            const int cnt = min(16, p.N - n);
+            for (int t = 0; t < cnt; ++t) dst[t] = (int8_t)(v[t >> 2] >> ((t & 3) * 8));
           }
         }
       }
@@ -460,25 +471,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmPa
     else if (gelu) body(std::true_type{}, std::false_type{});
     else if (has_bias) body(std::false_type{}, std::true_type{});
     else body(std::false_type{}, std::false_type{});
-    __syncthreads();
-    int8_t* Cz = (int8_t*)Cb + (int64_t)bz * p.sCb;
-    const bool vec_ok = ((p.sCm & 15) == 0) && ((((uintptr_t)Cz) & 15) == 0);
-    constexpr int SEGS = BN / 16;
-    for (int s = tid; s < BM * SEGS; s += NT) {
-      const int ml = s / SEGS, seg = s % SEGS;
-      const int m = m0 + ml, n = n0 + seg * 16;
-      if (m >= p.M || n >= p.N) continue;
-      const unsigned* src = (const unsigned*)(lds + ml * C_PITCH + seg * 16);
-      v4u v;
-      v[0] = src[0]; v[1] = src[1]; v[2] = src[2]; v[3] = src[3];
-      int8_t* dst = Cz + (int64_t)m * p.sCm + n;
-      if (vec_ok && n + 16 <= p.N) {
-        *(v4u*)dst = v;
-      } else {
-        const int cnt = min(16, p.N - n);
-        for (int t = 0; t < cnt; ++t) dst[t] = (int8_t)(v[t >> 2] >> ((t & 3) * 8));
-      }
-    }
   } else {
     // acc[i][j][r]: m = m0 + wm*WTM + i*32 + 8*(r/4) + 4*lhi + r%4;  n = n0 + wn*WTN + j*32 + lrow.
     constexpr int ESZ = OUTCLS == OUT32 ? 4 : 2;
@@ -525,9 +517,376 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_mfma_kernel(GemmPa
       else body(std::integral_constant<int, 4>{});
     }
   }
-#ifdef TI_TRACE
-  if (lane == 0 && blockIdx.x < 256) ti_trace_buf[(blockIdx.x * 4 + wave) * 8 + 6] = wall_clock64();
+}
+
+// ---- persistent ("stream") variant of the fast family --------------------------------------------
+//
+// One workgroup per CU slot walks a list of output tiles, and the global -> LDS pipeline does not
+// stop at a tile boundary: the k-tiles of all its tiles form one stream, the loads run NSTAGE-1
+// k-tiles ahead of the MFMAs, so the first operands of the next tile arrive while the epilogue of
+// the current one runs, and the epilogue's stores drain while the next tile computes.  What a
+// one-tile-per-workgroup launch pays per tile (first-load latency, the drain of its stores before
+// the workgroup can retire, the launch of its successor) is paid once per workgroup instead.
+//
+// Work list: the tiles*batch items are folded into 8 contiguous ranges, one per XCD (workgroup
+// b runs on XCD b % 8 when the grid is a multiple of 8), and the workgroups of an XCD interleave
+// over its range, so that tiles running at the same time share operand panels in that XCD's L2.
+//
+// Load counting.  vmcnt retires loads and stores in order.  The waits inside a k-loop name how
+// many younger operations may still be in flight; the epilogue's stores are younger than the
+// loads that were issued before it, so for the first NSTAGE-2 k-tiles after an epilogue the
+// count is raised by the number of store instructions STORES, which is exact because every store
+// is an unconditional buffer store (elements outside M x N are redirected out of the buffer's
+// range and dropped by the range check).  A count too small would only wait longer; 63 is the
+// counter's maximum.
+//
+// The epilogue touches no LDS: 4-byte and 2-byte outputs are stored straight from the MFMA layout
+// (32 consecutive n per row and instruction), int8 outputs exchange dwords between the two wave
+// halves so that every lane owns 16 consecutive bytes of a row.
+#ifndef TI_STREAM_STORE_AUX
+#define TI_STREAM_STORE_AUX 2
 #endif
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int SWZ, int NSTAGE, int OUTCLS, int OCC = 1>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3) / 4) void gemm_mfma_stream_kernel(GemmParams p) {
+  constexpr int NT = WAVES_M * WAVES_N * 64;
+  constexpr int CH = BK / 16;
+  constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int KS = BK / 32;
+  constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
+  constexpr int STAGE = A_BYTES + B_BYTES;
+  // int8 outputs: per wave a 32-row strip of its WTN output bytes (to turn the MFMA layout into
+  // long row segments) and WTN per-column fp32 terms
+  constexpr int STRIP = 32 * WTN, COLS = 4 * WTN;
+  constexpr int EPI_LDS = OUTCLS == OUT8 ? WAVES_M * WAVES_N * (STRIP + COLS) : 0;
+  constexpr int LDS_BYTES = NSTAGE * STAGE + EPI_LDS;
+  constexpr int DEPTH = NSTAGE - 1;
+  constexpr int ESZ = OUTCLS == OUT8 ? 1 : (OUTCLS == OUT32 ? 4 : 2);
+  constexpr int STORES = OUTCLS == OUT8 ? TM * TN : TM * TN * 16;  // store instructions per tile
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % 64 == 0, "tile shape");
+  static_assert(NSTAGE >= 3 && LDS_BYTES <= 160 * 1024, "LDS budget");
+
+  __shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+  // ---- this workgroup's items: ranks first, first + step, ... (count of them)
+  const int T = p.tiles_m * p.tiles_n;
+  const int W = T * p.batch;
+  int first, step, count;
+  {
+    const int G = (int)gridDim.x, b = (int)blockIdx.x;
+    if (G & 7) {
+      first = b;
+      step = G;
+      count = b < W ? (W - b + G - 1) / G : 0;
+    } else {
+      const int xcd = b & 7, l = b >> 3, nb = G >> 3;
+      const int per = W >> 3, rem = W & 7;
+      const int cnt = per + (xcd < rem ? 1 : 0);
+      first = xcd * per + min(xcd, rem) + l;
+      step = nb;
+      count = l < cnt ? (cnt - l + nb - 1) / nb : 0;
+    }
+    first = __builtin_amdgcn_readfirstlane(first);
+    step = __builtin_amdgcn_readfirstlane(step);
+    count = __builtin_amdgcn_readfirstlane(count);
+  }
+  if (count == 0) return;
+  auto locate = [&](int i, int& bz, int& m0, int& n0) {
+    const int g = first + i * step;
+    const int b_ = g / T;
+    int tm, tn;
+    tile_from_rank(p, g - b_ * T, tm, tn);
+    bz = __builtin_amdgcn_readfirstlane(b_);
+    m0 = __builtin_amdgcn_readfirstlane(tm * BM);
+    n0 = __builtin_amdgcn_readfirstlane(tn * BN);
+  };
+
+  const int lda = (int)p.sAm, ldb = (int)p.sBn;
+  const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+  const unsigned wave_slot = __builtin_amdgcn_readfirstlane(lds_base + wave * 1024);
+
+  // thread-constant offsets relative to the tile origin; the origin lives in the descriptors
+  TileLoader<BM, BK, NT, SWZ> la;
+  TileLoader<BN, BK, NT, SWZ> lb;
+  la.init(tid, 0, lda, p.K);
+  lb.init(tid, 0, ldb, p.K);
+  constexpr int A_IT = decltype(la)::IT, B_IT = decltype(lb)::IT;
+  constexpr int LOADS = A_IT + B_IT;
+  const int KT = (p.K + BK - 1) / BK;
+  const int KEND = KT * BK;
+  const int OOB = (int)0x80000000;
+
+  // ---- issue side of the stream: item i_issue, k offset k_issue, LDS stage st_issue
+  v4i rA, rB;
+  int i_issue = 0, k_issue = 0, st_issue = 0;
+  auto aim = [&](int i) {
+    if (i < count) {
+      int bz, m0, n0;
+      locate(i, bz, m0, n0);
+      // rows at or past M (N) and bytes past K of the last row read as zero
+      rA = make_rsrc(p.A + (int64_t)bz * p.sAb + (int64_t)m0 * lda, (p.M - 1 - m0) * lda + p.K);
+      rB = make_rsrc(p.B + (int64_t)bz * p.sBb + (int64_t)n0 * ldb, (p.N - 1 - n0) * ldb + p.K);
+    } else {
+      // past the last item: empty buffers, the loads write zeros into stages nobody reads, which
+      // keeps the number of loads in flight (and so the counts to wait for) constant
+      rA = make_rsrc(p.A, 0);
+      rB = make_rsrc(p.B, 0);
+    }
+  };
+  auto dma = [&](int d) {
+    if (d < A_IT) {
+      const unsigned dst = wave_slot + st_issue * STAGE + d * NT * 16;
+      dma16_to_lds(rA, (k_issue < la.klim[d]) ? la.voff[d] : OOB, k_issue, dst);
+    } else {
+      const int e = d - A_IT;
+      const unsigned dst = wave_slot + st_issue * STAGE + A_BYTES + e * NT * 16;
+      dma16_to_lds(rB, (k_issue < lb.klim[e]) ? lb.voff[e] : OOB, k_issue, dst);
+    }
+  };
+  auto dma_advance = [&]() {
+    k_issue += BK;
+    st_issue = (st_issue + 1 == NSTAGE) ? 0 : st_issue + 1;
+    if (k_issue >= KEND) {
+      k_issue = 0;
+      ++i_issue;
+      aim(i_issue);
+    }
+  };
+
+  v16i acc[TM][TN];
+  const int frow = lane & 31;
+  const int fsw = (frow >> SWZ) & (CH - 1);
+  const int fhalf = lane >> 5;
+  const int a_lane = (wm * WTM + frow) * BK;
+  const int b_lane = A_BYTES + (wn * WTN + frow) * BK;
+
+  v4i fa[2][TM], fb[2][TN];
+  auto load_frag = [&](const char* stage, int ks, int buf, int r) {
+    const int coff = ((ks * 2 + fhalf) ^ fsw) * 16;
+    if (r < TM) fa[buf][r] = *(const v4i*)(stage + a_lane + r * 32 * BK + coff);
+    else fb[buf][r - TM] = *(const v4i*)(stage + b_lane + (r - TM) * 32 * BK + coff);
+  };
+  auto mfma = [&](int buf, int u) {
+    const int i = u / TN, j = u % TN;
+    if constexpr (OUTCLS == OUT8)  // rows of the MFMA result = n (4 consecutive n per lane)
+      acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
+    else  // rows of the MFMA result = m, lanes run along n
+      acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
+  };
+  constexpr int NM = TM * TN, NR = TM + TN;
+  auto kstep = [&](int buf, const char* rd_stage, int rd_ks, bool do_read, int d0, int nd) {
+    int d = 0;
+#pragma unroll
+    for (int u = 0; u < NM; ++u) {
+      mfma(buf, u);
+      if (do_read) {
+#pragma unroll
+        for (int r = 0; r < NR; ++r)
+          if (r * NM / NR == u || (NM > NR && r == u)) {
+            if (NM > NR ? r == u : r * NM / NR == u) load_frag(rd_stage, rd_ks, buf ^ 1, r);
+          }
+      }
+      if (d < nd && (u + 1) * nd >= (d + 1) * NM) {
+        dma(d0 + d);
+        ++d;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  constexpr int PER_KS = (LOADS + KS - 1) / KS;
+  constexpr int LOADS_B = (LOADS - PER_KS * (KS - 1) > 0) ? LOADS - PER_KS * (KS - 1) : 0;
+  constexpr int LOADS_A = LOADS - LOADS_B;
+  constexpr int N_STEADY = LOADS * (DEPTH - 2) + LOADS_A;
+  constexpr int N_AFTER_STORES = (N_STEADY + STORES > 63) ? 63 : N_STEADY + STORES;
+
+  const EpiCtx e = make_epi(p);
+  const int lrow = lane & 31, lhi = lane >> 5;
+  const bool has_bias = e.bias_kind != TI_BIAS_NONE;
+
+  // ---- fill the pipeline
+  aim(0);
+#pragma unroll
+  for (int t = 0; t < DEPTH; ++t) {
+#pragma unroll
+    for (int d = 0; d < LOADS; ++d) dma(d);
+    dma_advance();
+  }
+  wait_loads_and_barrier<LOADS*(DEPTH - 1)>();
+
+  int st = 0;
+  for (int it = 0; it < count; ++it) {
+    int bz, m0, n0;
+    locate(it, bz, m0, n0);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+#ifdef TI_TRACE
+    const uint64_t tr_a = wall_clock64();
+    const uint64_t tr_ca = __builtin_readcyclecounter();
+#endif
+    // k-tile 0 of this item has landed: the barrier of the previous k-tile (or the one above) saw to it
+#pragma unroll
+    for (int r = 0; r < NR; ++r) load_frag(lds + st * STAGE, 0, 0, r);
+
+    for (int kt = 0; kt < KT; ++kt) {
+      const char* cur = lds + st * STAGE;
+      st = (st + 1 == NSTAGE) ? 0 : st + 1;
+#pragma unroll
+      for (int ks = 0; ks < KS - 1; ++ks) {
+        const int d0 = ks * PER_KS;
+        const int nd = (d0 + PER_KS <= LOADS_A) ? PER_KS : (LOADS_A - d0 > 0 ? LOADS_A - d0 : 0);
+        kstep(ks & 1, cur, ks + 1, true, d0, nd);
+      }
+      // all LDS reads of this k-tile are issued; the next k-tile must have landed before the
+      // barrier.  The stores of the previous item's epilogue are younger than that k-tile while
+      // it is one of those that were fetched before the epilogue.
+      if (it > 0 && kt < DEPTH - 1) wait_loads_and_barrier<N_AFTER_STORES>();
+      else wait_loads_and_barrier<N_STEADY>();
+      kstep((KS - 1) & 1, lds + st * STAGE, 0, kt + 1 < KT, LOADS_A, LOADS_B);
+      dma_advance();
+    }
+
+#ifdef TI_TRACE
+    const uint64_t tr_b = wall_clock64();
+    const uint64_t tr_cb = __builtin_readcyclecounter();
+#endif
+    // ---- epilogue: unconditional buffer stores, see the comment at the top
+    const int c_extent = ((p.M - 1) * (int)p.sCm + p.N) * ESZ;
+    const __amdgpu_buffer_rsrc_t rC =
+        __builtin_amdgcn_make_buffer_rsrc((char*)p.C + (int64_t)bz * p.sCb * ESZ, 0, c_extent, 0x00020000);
+    const int ldc = (int)p.sCm;
+    if constexpr (OUTCLS == OUT8) {
+      // acc[i][j][r]: m = m0 + wm*WTM + i*32 + lrow;  n = n0 + wn*WTN + j*32 + 8*(r/4) + 4*lhi + r%4.
+      // Quantise (clamp in fp32, then add 1.5*2^23: round to nearest even, int8 in the low byte),
+      // pack 4 consecutive n into a dword X[g], g = r/4.  Lanes l and l+32 hold the two halves of
+      // every 8-byte group of a row; swapping wave halves of (X0, X2) and of (X1, X3) leaves lane l
+      // with bytes 0..15 and lane l+32 with bytes 16..31 of the row's 32-byte segment.  A store
+      // of those would touch 32 rows with 32 bytes each; instead the wave writes its 32 x WTN strip
+      // to its own LDS area and reads it back with consecutive lanes along a row, so that a store
+      // instruction covers 1024/WTN rows with WTN consecutive bytes each.  16-byte segment s of
+      // strip row r lives at slot s ^ ((r / WRAP) % SEG), WRAP = rows per 256 bytes: conflict-free
+      // for the column-wise writes and the row-wise reads.  The area is private to the wave: no
+      // barrier, LDS operations of one wave execute in order.
+      constexpr int SEG = WTN / 16, RP = 64 / SEG, WRAP = 256 / WTN;
+      static_assert(32 % RP == 0 && 32 / RP == TN, "one read pass per 32-column block");
+      char* strip = lds + NSTAGE * STAGE + wave * (STRIP + COLS);
+      float* cols = (float*)(strip + STRIP);
+      const float q_floor = e.epilogue == TI_EPI_SCALE_RELU_I8 ? 0.0f : -128.0f;
+      const int w_swz = (lrow / WRAP) & (SEG - 1);
+      const int r_row = lane / SEG, r_seg = lane % SEG;
+      auto body = [&](auto gelu_tag, auto bias_tag) {
+        constexpr bool GELU = decltype(gelu_tag)::value;
+        constexpr bool BIAS = decltype(bias_tag)::value;
+        if constexpr (BIAS) {
+          // the wave's WTN per-column terms, once per tile (the loads come before this tile's
+          // stores, so waiting for them does not wait for a store)
+#pragma unroll
+          for (int c = lane; c < WTN; c += 64)
+            cols[c] = column_term_t<GELU ? TI_BIAS_F32 : TI_BIAS_I8>(e, min(n0 + wn * WTN + c, p.N - 1), GELU);
+        }
+        auto one = [&](int a, float col) -> unsigned {
+          float v = (float)a * e.alpha;
+          if constexpr (BIAS) v = col + v;
+          if constexpr (GELU) v = gelu_tanh_scaled(v, e.beta);
+          v = __builtin_amdgcn_fmed3f(v, q_floor, 127.0f);
+          return __float_as_uint(v + 12582912.0f);
+        };
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+            unsigned X[4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              v4f col = {0.f, 0.f, 0.f, 0.f};
+              if constexpr (BIAS) col = *(const v4f*)(cols + j * 32 + 8 * g + 4 * lhi);
+              const unsigned b0 = one(acc[i][j][4 * g + 0], col[0]), b1 = one(acc[i][j][4 * g + 1], col[1]);
+              const unsigned b2 = one(acc[i][j][4 * g + 2], col[2]), b3 = one(acc[i][j][4 * g + 3], col[3]);
+              X[g] = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u) | __builtin_amdgcn_perm(b3, b2, 0x04000c0cu);
+            }
+            const auto s02 = __builtin_amdgcn_permlane32_swap(X[0], X[2], false, false);
+            const auto s13 = __builtin_amdgcn_permlane32_swap(X[1], X[3], false, false);
+            v4u v;
+            v[0] = s02[0]; v[1] = s02[1]; v[2] = s13[0]; v[3] = s13[1];
+            *(v4u*)(strip + lrow * WTN + (((2 * j + lhi) ^ w_swz) * 16)) = v;
+          }
+#pragma unroll
+          for (int q = 0; q < TN; ++q) {
+            const int row = q * RP + r_row;
+            const v4u v = *(const v4u*)(strip + row * WTN + ((r_seg ^ ((row / WRAP) & (SEG - 1))) * 16));
+            const int m = m0 + wm * WTM + i * 32 + row;
+            const int n = n0 + wn * WTN + r_seg * 16;
+            const int off = (m < p.M && n < p.N) ? m * ldc + n : OOB;  // N % 16 == 0: a segment is in or out
+            __builtin_amdgcn_raw_buffer_store_b128(v, rC, off, 0, TI_STREAM_STORE_AUX);
+          }
+        }
+      };
+      const bool gelu = e.epilogue == TI_EPI_GELU_I8;
+      if (gelu && has_bias) body(std::true_type{}, std::true_type{});
+      else if (gelu) body(std::true_type{}, std::false_type{});
+      else if (has_bias) body(std::false_type{}, std::true_type{});
+      else body(std::false_type{}, std::false_type{});
+    } else {
+      // acc[i][j][r]: m = m0 + wm*WTM + i*32 + 8*(r/4) + 4*lhi + r%4;  n = n0 + wn*WTN + j*32 + lrow.
+      // KIND: 0 raw int32 (+ int32 bias), 1 scaled -> int32, 2 scaled -> fp32, 3 -> fp16, 4 -> bf16
+      auto body = [&](auto kind_tag) {
+        constexpr int KIND = decltype(kind_tag)::value;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const int n = n0 + wn * WTN + j * 32 + lrow;
+          const int nc = min(n, p.N - 1);
+          const float col = KIND == 0 ? 0.0f : column_term_t<KIND == 1 ? TI_BIAS_I32 : TI_BIAS_F32>(e, nc, false);
+          const int bias_i32 = (KIND == 0 && e.bias_kind == TI_BIAS_I32) ? ((const int*)e.bias)[nc] : 0;
+          const bool n_ok = n < p.N;
+#pragma unroll
+          for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int m = m0 + wm * WTM + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+              const int off = (n_ok && m < p.M) ? (m * ldc + n) * ESZ : OOB;
+              const int a = acc[i][j][r];
+              if constexpr (KIND == 0) {
+                __builtin_amdgcn_raw_buffer_store_b32((unsigned)a + (unsigned)bias_i32, rC, off, 0, 0);
+              } else {
+                float v = (float)a * e.alpha;
+                const float vb = col + v;
+                v = has_bias ? vb : v;
+                if constexpr (KIND == 1) __builtin_amdgcn_raw_buffer_store_b32((unsigned)q32(v, e.round_mode), rC, off, 0, 0);
+                else if constexpr (KIND == 2) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rC, off, 0, 0);
+                else if constexpr (KIND == 3) __builtin_amdgcn_raw_buffer_store_b16(f32_to_f16_bits(v), rC, off, 0, 0);
+                else __builtin_amdgcn_raw_buffer_store_b16(f32_to_bf16_bits(v), rC, off, 0, 0);
+              }
+            }
+          }
+        }
+      };
+      if constexpr (OUTCLS == OUT32) {
+        if (e.epilogue == TI_EPI_I32) body(std::integral_constant<int, 0>{});
+        else if (e.epilogue == TI_EPI_SCALE_I32) body(std::integral_constant<int, 1>{});
+        else body(std::integral_constant<int, 2>{});
+      } else {
+        if (p.out_dtype == TI_F16) body(std::integral_constant<int, 3>{});
+        else body(std::integral_constant<int, 4>{});
+      }
+    }
+#ifdef TI_TRACE
+    if (lane == 0 && blockIdx.x < 256 && it == 2) {
+      unsigned long long* tr = ti_trace_buf + (blockIdx.x * 4 + (wave & 3)) * 8;
+      tr[0] = tr_a; tr[1] = tr_b; tr[2] = wall_clock64(); tr[3] = tr_cb - tr_ca; tr[4] = __builtin_readcyclecounter() - tr_cb;
+    }
+#endif
+  }
+  // the trailing (empty-buffer) loads still write zeros into LDS: they must land before the
+  // workgroup's LDS is handed to another one
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 // ---- gather family -----------------------------------------------------------------------------
@@ -742,6 +1101,7 @@ struct Config {
   int bm, bn, bk, threads;
   bool fast;       // needs the aligned K-contiguous layout
   bool skinny = false;  // gemm_skinny_kernel: M <= 64, grid over 16-row slabs of B
+  int stream_occ = 0;   // > 0: gemm_mfma_stream_kernel, this many workgroups per CU walk the tile list
 };
 
 #define TI_FAST(BM, BN, BK, WM, WN, SWZ, NS)                                              \
@@ -753,21 +1113,44 @@ struct Config {
         BM, BN, BK, WM * WN * 64, true                                                    \
   }
 
+#define TI_STREAM(BM, BN, BK, WM, WN, SWZ, NS, OCC)                                        \
+  {                                                                                       \
+    "stream_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN "_s" #SWZ "_p" #NS "_o" #OCC,            \
+        {gemm_mfma_stream_kernel<BM, BN, BK, WM, WN, SWZ, NS, OUT8, OCC>,                   \
+         gemm_mfma_stream_kernel<BM, BN, BK, WM, WN, SWZ, NS, OUT32, OCC>,                  \
+         gemm_mfma_stream_kernel<BM, BN, BK, WM, WN, SWZ, NS, OUT16, OCC>},                 \
+        BM, BN, BK, WM * WN * 64, true, false, OCC                                        \
+  }
+
+enum ConfigId {
+  CFG_GATHER = 0,
+  CFG_TILE_256x128,   // one tile per workgroup: any output layout the fast loads allow
+  CFG_TILE_256x256,
+  CFG_TILE_128x128,
+  CFG_TILE_64x64,
+  CFG_SKINNY_16,
+  CFG_SKINNY_32,
+  CFG_SKINNY_64,
+  CFG_STREAM_256x256,       // persistent: row-major, 16-byte aligned outputs
+  CFG_STREAM_256x256_WIDE,  // waves 128 columns wide: int8 rows leave as whole 128-byte lines
+  CFG_STREAM_256x128,
+  CFG_STREAM_128x128,
+};
+
 static const Config g_configs[] = {
     {"gather_64x64x32", {gemm_gather_kernel<OUT8>, gemm_gather_kernel<OUT32>, gemm_gather_kernel<OUT16>}, 64, 64, 32, 256, false},
-    TI_FAST(256, 128, 128, 2, 2, 1, 3),  // 1
-    TI_FAST(256, 128, 128, 4, 2, 1, 3),  // 2
-    TI_FAST(256, 128, 128, 2, 4, 1, 3),  // 3
-    TI_FAST(256, 256, 64, 2, 4, 2, 4),   // 4
-    TI_FAST(256, 256, 64, 4, 2, 2, 4),   // 5
-    TI_FAST(128, 128, 64, 2, 2, 2, 4),   // 6
-    TI_FAST(128, 128, 128, 2, 2, 1, 3),  // 7
-    TI_FAST(64, 64, 128, 2, 2, 1, 3),    // 8
-    {"skinny_m16_slab16", {gemm_skinny_kernel<OUT8, 1>, gemm_skinny_kernel<OUT32, 1>, gemm_skinny_kernel<OUT16, 1>}, 16, 16, 64, 512, true, true},  // 9
-    {"skinny_m32_slab16", {gemm_skinny_kernel<OUT8, 2>, gemm_skinny_kernel<OUT32, 2>, gemm_skinny_kernel<OUT16, 2>}, 32, 16, 64, 512, true, true},  // 10
-    {"skinny_m64_slab16", {gemm_skinny_kernel<OUT8, 4>, gemm_skinny_kernel<OUT32, 4>, gemm_skinny_kernel<OUT16, 4>}, 64, 16, 64, 512, true, true},  // 11
+    TI_FAST(256, 128, 128, 2, 2, 1, 3),
+    TI_FAST(256, 256, 64, 2, 4, 2, 4),
+    TI_FAST(128, 128, 64, 2, 2, 2, 4),
+    TI_FAST(64, 64, 128, 2, 2, 1, 3),
+    {"skinny_m16_slab16", {gemm_skinny_kernel<OUT8, 1>, gemm_skinny_kernel<OUT32, 1>, gemm_skinny_kernel<OUT16, 1>}, 16, 16, 64, 512, true, true},
+    {"skinny_m32_slab16", {gemm_skinny_kernel<OUT8, 2>, gemm_skinny_kernel<OUT32, 2>, gemm_skinny_kernel<OUT16, 2>}, 32, 16, 64, 512, true, true},
+    {"skinny_m64_slab16", {gemm_skinny_kernel<OUT8, 4>, gemm_skinny_kernel<OUT32, 4>, gemm_skinny_kernel<OUT16, 4>}, 64, 16, 64, 512, true, true},
+    TI_STREAM(256, 256, 64, 2, 4, 2, 4, 1),
+    TI_STREAM(256, 256, 64, 4, 2, 2, 3, 1),
+    TI_STREAM(256, 128, 128, 2, 2, 1, 3, 1),
+    TI_STREAM(128, 128, 64, 2, 2, 2, 3, 2),
 };
-static const int SKINNY_CFG = 9;
 static const int g_num_configs = (int)(sizeof(g_configs) / sizeof(g_configs[0]));
 
 static int out_class(int out_dtype) {
@@ -788,35 +1171,50 @@ static bool fast_eligible(const GemmParams& p) {
   if (out_class(p.out_dtype) == OUT8 && p.sCn != 1) return false;
   // 32-bit byte offsets inside one batch slice, including the rows a ragged last tile touches
   const int64_t lim = (int64_t)1 << 31;
-  if (((int64_t)p.M + 256) * p.sAm + p.K >= lim) return false;
-  if (((int64_t)p.N + 256) * p.sBn + p.K >= lim) return false;
+  if (((int64_t)p.M + 512) * p.sAm + p.K >= lim) return false;
+  if (((int64_t)p.N + 512) * p.sBn + p.K >= lim) return false;
+  return true;
+}
+
+// The stream kernels store through range-checked buffer descriptors with 32-bit offsets and, for
+// int8, whole 16-byte segments only.
+static bool stream_eligible(const GemmParams& p) {
+  if (!fast_eligible(p)) return false;
+  if (p.sCn != 1 || p.sCm < p.N || p.sCb < 0) return false;
+  const int oc = out_class(p.out_dtype);
+  const int esz = oc == OUT8 ? 1 : (oc == OUT32 ? 4 : 2);
+  if (((int64_t)p.M * p.sCm + p.N) * esz >= ((int64_t)1 << 31)) return false;
+  if ((uintptr_t)p.C % esz) return false;
+  if (oc == OUT8 && ((p.N & 15) || (p.sCm & 15) || (p.sCb & 15) || ((uintptr_t)p.C & 15))) return false;
   return true;
 }
 
 // Tile choice: score = (measured relative efficiency of the tile class) x (fraction of the
 // 256 CUs kept busy over all rounds of workgroups) x (fraction of the tiles' area that is real
-// output).  Within a class the wave arrangement depends on the output width: 4-byte outputs
-// store straight from the MFMA layout and prefer waves stacked along M, int8 outputs go through
-// the LDS staging; the preferences were measured with weights streamed from HBM.
+// output).  The class efficiencies were measured with weights streamed from HBM.  Outputs the
+// persistent kernels can store (row-major, aligned) go to them; the rest to the one-tile kernels.
 static int pick_config(const GemmParams& p) {
-  if (!fast_eligible(p)) return 0;
-  if (p.M <= 64) return SKINNY_CFG + (p.M > 16) + (p.M > 32);
-  const bool wide_out = out_class(p.out_dtype) != OUT8;
+  if (!fast_eligible(p)) return CFG_GATHER;
+  if (p.M <= 64) return CFG_SKINNY_16 + (p.M > 16) + (p.M > 32);
+  const bool stream = stream_eligible(p);
+  // short K, int8 out: the epilogue and its stores dominate, whole-line stores pay
+  const bool wide = out_class(p.out_dtype) == OUT8 && p.K <= 256;
   struct Cand { int cfg; double base; };
   const Cand cands[] = {
-      {wide_out ? 5 : 4, 1.00},
-      {wide_out ? 2 : (p.epilogue == TI_EPI_GELU_I8 ? 3 : 1), 0.90},
-      {6, 0.78},
-      {8, 0.50},
+      {stream ? (wide ? CFG_STREAM_256x256_WIDE : CFG_STREAM_256x256) : CFG_TILE_256x256, 1.00},
+      {stream ? CFG_STREAM_256x128 : CFG_TILE_256x128, 0.90},
+      {stream ? CFG_STREAM_128x128 : CFG_TILE_128x128, 0.78},
+      {CFG_TILE_64x64, 0.50},
   };
-  int best = 8;
+  int best = CFG_TILE_64x64;
   double best_score = -1.0;
   for (const Cand& c : cands) {
     const Config& k = g_configs[c.cfg];
+    const int slots = 256 * (k.stream_occ > 1 ? k.stream_occ : 1);
     const int64_t tm = (p.M + k.bm - 1) / k.bm, tn = (p.N + k.bn - 1) / k.bn;
     const int64_t tiles = tm * tn * p.batch;
-    const int64_t rounds = (tiles + 255) / 256;
-    const double busy = (double)tiles / (double)(rounds * 256);
+    const int64_t rounds = (tiles + slots - 1) / slots;
+    const double busy = (double)tiles / (double)(rounds * slots);
     const double area = ((double)p.M * p.N) / ((double)(tm * k.bm) * (double)(tn * k.bn));
     const double score = c.base * busy * area;
     if (score > best_score) best_score = score, best = c.cfg;
@@ -880,11 +1278,12 @@ static int run(GemmParams p, int config, hipStream_t stream) {
   // the fast kernels quantise to int8 with round-half-even only; the truncating test switch runs
   // on the gather kernel
   const bool trunc8 = p.round_mode == TI_ROUND_TRUNC && out_class(p.out_dtype) == OUT8;
-  if (config < 0) config = (trunc8 && p.M > 64) ? 0 : pick_config(p);
+  if (config < 0) config = (trunc8 && p.M > 64) ? CFG_GATHER : pick_config(p);
   if (config >= g_num_configs) return fail(TI_E_COMBO, "config %d out of range", config);
   const Config& k = g_configs[config];
   if (k.fast && !k.skinny && trunc8) return fail(TI_E_COMBO, "config %s does not implement TI_ROUND_TRUNC for int8 outputs", k.name);
   if (k.fast && !fast_eligible(p)) return fail(TI_E_COMBO, "config %s needs K-contiguous 16-byte aligned operands", k.name);
+  if (k.stream_occ && !stream_eligible(p)) return fail(TI_E_COMBO, "config %s needs a row-major output with 16-byte aligned rows", k.name);
   if (k.skinny) {
     if (p.M > k.bm) return fail(TI_E_COMBO, "config %s needs M <= %d", k.name, k.bm);
     // enough waves to fill the chip: split K between the waves of a workgroup when there are few slabs
@@ -903,8 +1302,16 @@ static int run(GemmParams p, int config, hipStream_t stream) {
   p.tiles_n = (p.N + k.bn - 1) / k.bn;
   if ((int64_t)p.tiles_m * p.tiles_n > 0x7fffffff) return fail(TI_E_SHAPE, "too many tiles");
   p.group_m = pick_group_m(p, k);
-  dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)p.batch, 1);
   g_last_config = config;
+  if (k.stream_occ) {
+    const int64_t items = (int64_t)p.tiles_m * p.tiles_n * p.batch;
+    if (items > 0x7fffffff) return fail(TI_E_SHAPE, "too many tiles");
+    int64_t g = items < 256 * k.stream_occ ? items : 256 * k.stream_occ;
+    if (g >= 8) g &= ~(int64_t)7;  // a multiple of 8 keeps workgroup b on XCD b % 8
+    k.fn[out_class(p.out_dtype)]<<<dim3((unsigned)g), dim3(k.threads), 0, stream>>>(p);
+    return launch_status(k.name);
+  }
+  dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)p.batch, 1);
   k.fn[out_class(p.out_dtype)]<<<grid, dim3(k.threads), 0, stream>>>(p);
   return launch_status(k.name);
 }
