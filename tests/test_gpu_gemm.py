@@ -26,7 +26,7 @@ def _configs(M=1, N=None, out8=False):
     def fits(nm):  # "skinny_m<rows>_..." configurations take at most <rows> activation rows
         if nm.startswith("skinny"):
             return M <= int(nm.split("_")[1][1:])
-        if nm.startswith("stream") and out8:
+        if nm.startswith(("stream", "ws_")) and out8:
             return N is not None and N % 16 == 0
         return True
     return [(i, nm) for i, nm in out if fits(nm)]
@@ -200,7 +200,7 @@ def test_stream_configs_many_tiles_per_workgroup(B, M, N, K):
     wantf = O.bmm_s8t_s8n_f32t(a, b, alpha)
     ran = 0
     for cfg, name in _configs(M, N, out8=True):
-        if not name.startswith("stream"):
+        if not name.startswith(("stream", "ws_")):
             continue
         ran += 1
         assert np.array_equal(cpu(bmm.bmm_s8t_s8n_s32t(ga, gb, _config=cfg)), want32), name

@@ -519,6 +519,142 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
   }
 }
 
+// ---- epilogue of the persistent kernels ----------------------------------------------------------
+// Stores one wave's (TM*32) x (TN*32) block of accumulators, whose first row / column in the
+// output are mw / nw, through an unconditional, range-checked buffer store per element group
+// (elements outside M x N are redirected out of the buffer's range and dropped), so that the
+// number of store instructions per tile is a compile-time constant.  `strip` is the wave's private
+// LDS area (int8 outputs only): 32*WTN bytes for the row strip plus WTN floats of column terms.
+#ifndef TI_STREAM_STORE_AUX
+#define TI_STREAM_STORE_AUX 2  // nt: the outputs are streamed, keep the operand panels in L2
+#endif
+template <int TM, int TN, int OUTCLS>
+__device__ __forceinline__ void stream_epilogue(const GemmParams& p, const EpiCtx& e, v16i (&acc)[TM][TN], int bz,
+                                                int mw, int nw, char* strip, int lane) {
+  constexpr int WTN = TN * 32;
+  constexpr int ESZ = OUTCLS == OUT8 ? 1 : (OUTCLS == OUT32 ? 4 : 2);
+  const int OOB = (int)0x80000000;
+  const int lrow = lane & 31, lhi = lane >> 5;
+  const bool has_bias = e.bias_kind != TI_BIAS_NONE;
+  const int c_extent = ((p.M - 1) * (int)p.sCm + p.N) * ESZ;
+  const __amdgpu_buffer_rsrc_t rC =
+      __builtin_amdgcn_make_buffer_rsrc((char*)p.C + (int64_t)bz * p.sCb * ESZ, 0, c_extent, 0x00020000);
+  const int ldc = (int)p.sCm;
+  if constexpr (OUTCLS == OUT8) {
+    // acc[i][j][r]: m = mw + i*32 + lrow;  n = nw + j*32 + 8*(r/4) + 4*lhi + r%4.
+    // Quantise (clamp in fp32, then add 1.5*2^23: round to nearest even, int8 in the low byte),
+    // pack 4 consecutive n into a dword X[g], g = r/4.  Lanes l and l+32 hold the two halves of
+    // every 8-byte group of a row; swapping wave halves of (X0, X2) and of (X1, X3) leaves lane l
+    // with bytes 0..15 and lane l+32 with bytes 16..31 of the row's 32-byte segment.  A store
+    // of those would touch 32 rows with 32 bytes each; instead the wave writes its 32 x WTN strip
+    // to its own LDS area and reads it back with consecutive lanes along a row, so that a store
+    // instruction covers 1024/WTN rows with WTN consecutive bytes each.  16-byte segment s of
+    // strip row r lives at slot s ^ ((r / WRAP) % SEG), WRAP = rows per 256 bytes: conflict-free
+    // for the column-wise writes and the row-wise reads.  The area is private to the wave: no
+    // barrier, LDS operations of one wave execute in order.
+    constexpr int SEG = WTN / 16, RP = 64 / SEG, WRAP = 256 / WTN;
+    static_assert(32 % RP == 0 && 32 / RP == TN, "one read pass per 32-column block");
+    float* cols = (float*)(strip + 32 * WTN);
+    const float q_floor = e.epilogue == TI_EPI_SCALE_RELU_I8 ? 0.0f : -128.0f;
+    const int w_swz = (lrow / WRAP) & (SEG - 1);
+    const int r_row = lane / SEG, r_seg = lane % SEG;
+    auto body = [&](auto gelu_tag, auto bias_tag) {
+      constexpr bool GELU = decltype(gelu_tag)::value;
+      constexpr bool BIAS = decltype(bias_tag)::value;
+      if constexpr (BIAS) {
+        // the wave's WTN per-column terms, once per tile (the loads come before this tile's
+        // stores, so waiting for them does not wait for a store)
+#pragma unroll
+        for (int c = lane; c < WTN; c += 64)
+          cols[c] = column_term_t<GELU ? TI_BIAS_F32 : TI_BIAS_I8>(e, min(nw + c, p.N - 1), GELU);
+      }
+      auto one = [&](int a, float col) -> unsigned {
+        float v = (float)a * e.alpha;
+        if constexpr (BIAS) v = col + v;
+        if constexpr (GELU) v = gelu_tanh_scaled(v, e.beta);
+        v = __builtin_amdgcn_fmed3f(v, q_floor, 127.0f);
+        return __float_as_uint(v + 12582912.0f);
+      };
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          unsigned X[4];
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            v4f col = {0.f, 0.f, 0.f, 0.f};
+            if constexpr (BIAS) col = *(const v4f*)(cols + j * 32 + 8 * g + 4 * lhi);
+            const unsigned b0 = one(acc[i][j][4 * g + 0], col[0]), b1 = one(acc[i][j][4 * g + 1], col[1]);
+            const unsigned b2 = one(acc[i][j][4 * g + 2], col[2]), b3 = one(acc[i][j][4 * g + 3], col[3]);
+            X[g] = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u) | __builtin_amdgcn_perm(b3, b2, 0x04000c0cu);
+          }
+          const auto s02 = __builtin_amdgcn_permlane32_swap(X[0], X[2], false, false);
+          const auto s13 = __builtin_amdgcn_permlane32_swap(X[1], X[3], false, false);
+          v4u v;
+          v[0] = s02[0]; v[1] = s02[1]; v[2] = s13[0]; v[3] = s13[1];
+          *(v4u*)(strip + lrow * WTN + (((2 * j + lhi) ^ w_swz) * 16)) = v;
+        }
+#pragma unroll
+        for (int q = 0; q < TN; ++q) {
+          const int row = q * RP + r_row;
+          const v4u v = *(const v4u*)(strip + row * WTN + ((r_seg ^ ((row / WRAP) & (SEG - 1))) * 16));
+          const int m = mw + i * 32 + row;
+          const int n = nw + r_seg * 16;
+          const int off = (m < p.M && n < p.N) ? m * ldc + n : OOB;  // N % 16 == 0: a segment is in or out
+          __builtin_amdgcn_raw_buffer_store_b128(v, rC, off, 0, TI_STREAM_STORE_AUX);
+        }
+      }
+    };
+    const bool gelu = e.epilogue == TI_EPI_GELU_I8;
+    if (gelu && has_bias) body(std::true_type{}, std::true_type{});
+    else if (gelu) body(std::true_type{}, std::false_type{});
+    else if (has_bias) body(std::false_type{}, std::true_type{});
+    else body(std::false_type{}, std::false_type{});
+  } else {
+    // acc[i][j][r]: m = mw + i*32 + 8*(r/4) + 4*lhi + r%4;  n = nw + j*32 + lrow.
+    // KIND: 0 raw int32 (+ int32 bias), 1 scaled -> int32, 2 scaled -> fp32, 3 -> fp16, 4 -> bf16
+    auto body = [&](auto kind_tag) {
+      constexpr int KIND = decltype(kind_tag)::value;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int n = nw + j * 32 + lrow;
+        const int nc = min(n, p.N - 1);
+        const float col = KIND == 0 ? 0.0f : column_term_t<KIND == 1 ? TI_BIAS_I32 : TI_BIAS_F32>(e, nc, false);
+        const int bias_i32 = (KIND == 0 && e.bias_kind == TI_BIAS_I32) ? ((const int*)e.bias)[nc] : 0;
+        const bool n_ok = n < p.N;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int m = mw + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
+            const int off = (n_ok && m < p.M) ? (m * ldc + n) * ESZ : OOB;
+            const int a = acc[i][j][r];
+            if constexpr (KIND == 0) {
+              __builtin_amdgcn_raw_buffer_store_b32((unsigned)a + (unsigned)bias_i32, rC, off, 0, 0);
+            } else {
+              float v = (float)a * e.alpha;
+              const float vb = col + v;
+              v = has_bias ? vb : v;
+              if constexpr (KIND == 1) __builtin_amdgcn_raw_buffer_store_b32((unsigned)q32(v, e.round_mode), rC, off, 0, 0);
+              else if constexpr (KIND == 2) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rC, off, 0, 0);
+              else if constexpr (KIND == 3) __builtin_amdgcn_raw_buffer_store_b16(f32_to_f16_bits(v), rC, off, 0, 0);
+              else __builtin_amdgcn_raw_buffer_store_b16(f32_to_bf16_bits(v), rC, off, 0, 0);
+            }
+          }
+        }
+      }
+    };
+    if constexpr (OUTCLS == OUT32) {
+      if (e.epilogue == TI_EPI_I32) body(std::integral_constant<int, 0>{});
+      else if (e.epilogue == TI_EPI_SCALE_I32) body(std::integral_constant<int, 1>{});
+      else body(std::integral_constant<int, 2>{});
+    } else {
+      if (p.out_dtype == TI_F16) body(std::integral_constant<int, 3>{});
+      else body(std::integral_constant<int, 4>{});
+    }
+  }
+}
+
 // ---- persistent ("stream") variant of the fast family --------------------------------------------
 //
 // One workgroup per CU slot walks a list of output tiles, and the global -> LDS pipeline does not
@@ -543,9 +679,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
 // The epilogue touches no LDS: 4-byte and 2-byte outputs are stored straight from the MFMA layout
 // (32 consecutive n per row and instruction), int8 outputs exchange dwords between the two wave
 // halves so that every lane owns 16 consecutive bytes of a row.
-#ifndef TI_STREAM_STORE_AUX
-#define TI_STREAM_STORE_AUX 2
-#endif
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int SWZ, int NSTAGE, int OUTCLS, int OCC = 1>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3) / 4) void gemm_mfma_stream_kernel(GemmParams p) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
@@ -561,7 +694,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
   constexpr int EPI_LDS = OUTCLS == OUT8 ? WAVES_M * WAVES_N * (STRIP + COLS) : 0;
   constexpr int LDS_BYTES = NSTAGE * STAGE + EPI_LDS;
   constexpr int DEPTH = NSTAGE - 1;
-  constexpr int ESZ = OUTCLS == OUT8 ? 1 : (OUTCLS == OUT32 ? 4 : 2);
   constexpr int STORES = OUTCLS == OUT8 ? TM * TN : TM * TN * 16;  // store instructions per tile
   static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % 64 == 0, "tile shape");
   static_assert(NSTAGE >= 3 && LDS_BYTES <= 160 * 1024, "LDS budget");
@@ -705,8 +837,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
   constexpr int N_AFTER_STORES = (N_STEADY + STORES > 63) ? 63 : N_STEADY + STORES;
 
   const EpiCtx e = make_epi(p);
-  const int lrow = lane & 31, lhi = lane >> 5;
-  const bool has_bias = e.bias_kind != TI_BIAS_NONE;
 
   // ---- fill the pipeline
   aim(0);
@@ -758,125 +888,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
     const uint64_t tr_b = wall_clock64();
     const uint64_t tr_cb = __builtin_readcyclecounter();
 #endif
-    // ---- epilogue: unconditional buffer stores, see the comment at the top
-    const int c_extent = ((p.M - 1) * (int)p.sCm + p.N) * ESZ;
-    const __amdgpu_buffer_rsrc_t rC =
-        __builtin_amdgcn_make_buffer_rsrc((char*)p.C + (int64_t)bz * p.sCb * ESZ, 0, c_extent, 0x00020000);
-    const int ldc = (int)p.sCm;
-    if constexpr (OUTCLS == OUT8) {
-      // acc[i][j][r]: m = m0 + wm*WTM + i*32 + lrow;  n = n0 + wn*WTN + j*32 + 8*(r/4) + 4*lhi + r%4.
-      // Quantise (clamp in fp32, then add 1.5*2^23: round to nearest even, int8 in the low byte),
-      // pack 4 consecutive n into a dword X[g], g = r/4.  Lanes l and l+32 hold the two halves of
-      // every 8-byte group of a row; swapping wave halves of (X0, X2) and of (X1, X3) leaves lane l
-      // with bytes 0..15 and lane l+32 with bytes 16..31 of the row's 32-byte segment.  A store
-      // of those would touch 32 rows with 32 bytes each; instead the wave writes its 32 x WTN strip
-      // to its own LDS area and reads it back with consecutive lanes along a row, so that a store
-      // instruction covers 1024/WTN rows with WTN consecutive bytes each.  16-byte segment s of
-      // strip row r lives at slot s ^ ((r / WRAP) % SEG), WRAP = rows per 256 bytes: conflict-free
-      // for the column-wise writes and the row-wise reads.  The area is private to the wave: no
-      // barrier, LDS operations of one wave execute in order.
-      constexpr int SEG = WTN / 16, RP = 64 / SEG, WRAP = 256 / WTN;
-      static_assert(32 % RP == 0 && 32 / RP == TN, "one read pass per 32-column block");
-      char* strip = lds + NSTAGE * STAGE + wave * (STRIP + COLS);
-      float* cols = (float*)(strip + STRIP);
-      const float q_floor = e.epilogue == TI_EPI_SCALE_RELU_I8 ? 0.0f : -128.0f;
-      const int w_swz = (lrow / WRAP) & (SEG - 1);
-      const int r_row = lane / SEG, r_seg = lane % SEG;
-      auto body = [&](auto gelu_tag, auto bias_tag) {
-        constexpr bool GELU = decltype(gelu_tag)::value;
-        constexpr bool BIAS = decltype(bias_tag)::value;
-        if constexpr (BIAS) {
-          // the wave's WTN per-column terms, once per tile (the loads come before this tile's
-          // stores, so waiting for them does not wait for a store)
-#pragma unroll
-          for (int c = lane; c < WTN; c += 64)
-            cols[c] = column_term_t<GELU ? TI_BIAS_F32 : TI_BIAS_I8>(e, min(n0 + wn * WTN + c, p.N - 1), GELU);
-        }
-        auto one = [&](int a, float col) -> unsigned {
-          float v = (float)a * e.alpha;
-          if constexpr (BIAS) v = col + v;
-          if constexpr (GELU) v = gelu_tanh_scaled(v, e.beta);
-          v = __builtin_amdgcn_fmed3f(v, q_floor, 127.0f);
-          return __float_as_uint(v + 12582912.0f);
-        };
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-#pragma unroll
-          for (int j = 0; j < TN; ++j) {
-            unsigned X[4];
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-              v4f col = {0.f, 0.f, 0.f, 0.f};
-              if constexpr (BIAS) col = *(const v4f*)(cols + j * 32 + 8 * g + 4 * lhi);
-              const unsigned b0 = one(acc[i][j][4 * g + 0], col[0]), b1 = one(acc[i][j][4 * g + 1], col[1]);
-              const unsigned b2 = one(acc[i][j][4 * g + 2], col[2]), b3 = one(acc[i][j][4 * g + 3], col[3]);
-              X[g] = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u) | __builtin_amdgcn_perm(b3, b2, 0x04000c0cu);
-            }
-            const auto s02 = __builtin_amdgcn_permlane32_swap(X[0], X[2], false, false);
-            const auto s13 = __builtin_amdgcn_permlane32_swap(X[1], X[3], false, false);
-            v4u v;
-            v[0] = s02[0]; v[1] = s02[1]; v[2] = s13[0]; v[3] = s13[1];
-            *(v4u*)(strip + lrow * WTN + (((2 * j + lhi) ^ w_swz) * 16)) = v;
-          }
-#pragma unroll
-          for (int q = 0; q < TN; ++q) {
-            const int row = q * RP + r_row;
-            const v4u v = *(const v4u*)(strip + row * WTN + ((r_seg ^ ((row / WRAP) & (SEG - 1))) * 16));
-            const int m = m0 + wm * WTM + i * 32 + row;
-            const int n = n0 + wn * WTN + r_seg * 16;
-            const int off = (m < p.M && n < p.N) ? m * ldc + n : OOB;  // N % 16 == 0: a segment is in or out
-            __builtin_amdgcn_raw_buffer_store_b128(v, rC, off, 0, TI_STREAM_STORE_AUX);
-          }
-        }
-      };
-      const bool gelu = e.epilogue == TI_EPI_GELU_I8;
-      if (gelu && has_bias) body(std::true_type{}, std::true_type{});
-      else if (gelu) body(std::true_type{}, std::false_type{});
-      else if (has_bias) body(std::false_type{}, std::true_type{});
-      else body(std::false_type{}, std::false_type{});
-    } else {
-      // acc[i][j][r]: m = m0 + wm*WTM + i*32 + 8*(r/4) + 4*lhi + r%4;  n = n0 + wn*WTN + j*32 + lrow.
-      // KIND: 0 raw int32 (+ int32 bias), 1 scaled -> int32, 2 scaled -> fp32, 3 -> fp16, 4 -> bf16
-      auto body = [&](auto kind_tag) {
-        constexpr int KIND = decltype(kind_tag)::value;
-#pragma unroll
-        for (int j = 0; j < TN; ++j) {
-          const int n = n0 + wn * WTN + j * 32 + lrow;
-          const int nc = min(n, p.N - 1);
-          const float col = KIND == 0 ? 0.0f : column_term_t<KIND == 1 ? TI_BIAS_I32 : TI_BIAS_F32>(e, nc, false);
-          const int bias_i32 = (KIND == 0 && e.bias_kind == TI_BIAS_I32) ? ((const int*)e.bias)[nc] : 0;
-          const bool n_ok = n < p.N;
-#pragma unroll
-          for (int i = 0; i < TM; ++i) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const int m = m0 + wm * WTM + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
-              const int off = (n_ok && m < p.M) ? (m * ldc + n) * ESZ : OOB;
-              const int a = acc[i][j][r];
-              if constexpr (KIND == 0) {
-                __builtin_amdgcn_raw_buffer_store_b32((unsigned)a + (unsigned)bias_i32, rC, off, 0, 0);
-              } else {
-                float v = (float)a * e.alpha;
-                const float vb = col + v;
-                v = has_bias ? vb : v;
-                if constexpr (KIND == 1) __builtin_amdgcn_raw_buffer_store_b32((unsigned)q32(v, e.round_mode), rC, off, 0, 0);
-                else if constexpr (KIND == 2) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rC, off, 0, 0);
-                else if constexpr (KIND == 3) __builtin_amdgcn_raw_buffer_store_b16(f32_to_f16_bits(v), rC, off, 0, 0);
-                else __builtin_amdgcn_raw_buffer_store_b16(f32_to_bf16_bits(v), rC, off, 0, 0);
-              }
-            }
-          }
-        }
-      };
-      if constexpr (OUTCLS == OUT32) {
-        if (e.epilogue == TI_EPI_I32) body(std::integral_constant<int, 0>{});
-        else if (e.epilogue == TI_EPI_SCALE_I32) body(std::integral_constant<int, 1>{});
-        else body(std::integral_constant<int, 2>{});
-      } else {
-        if (p.out_dtype == TI_F16) body(std::integral_constant<int, 3>{});
-        else body(std::integral_constant<int, 4>{});
-      }
-    }
+    // ---- epilogue
+    stream_epilogue<TM, TN, OUTCLS>(p, e, acc, bz, m0 + wm * WTM, n0 + wn * WTN,
+                                    lds + NSTAGE * STAGE + wave * (STRIP + COLS), lane);
 #ifdef TI_TRACE
     if (lane == 0 && blockIdx.x < 256 && it == 2) {
       unsigned long long* tr = ti_trace_buf + (blockIdx.x * 4 + (wave & 3)) * 8;
@@ -887,6 +901,207 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
   // the trailing (empty-buffer) loads still write zeros into LDS: they must land before the
   // workgroup's LDS is handed to another one
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+// ---- wave-specialised persistent kernel -------------------------------------------------------
+//
+// A wave that issues a 16-byte-per-lane load is held for about 64 cycles by the address path, and
+// while it is held it issues no MFMA: with the loads spread over the MFMA waves the matrix pipe
+// idles about a quarter of the k-loop.  Here the two jobs belong to different waves of the
+// workgroup.  PW producer waves do nothing but the global -> LDS loads of the k-tile stream
+// (tile list, descriptors, NSTAGE-1 k-tiles ahead, as in gemm_mfma_stream_kernel); the
+// WAVES_M x WAVES_N consumer waves only read fragments from LDS and issue MFMAs, then run the
+// epilogue.  With one consumer and one producer wave per SIMD the producer's address phases
+// overlap the consumer's MFMAs.
+//
+// Hand-over, one s_barrier per k-tile joined by all waves.  Iteration g (stream k-tile g):
+//   producer: issue the loads of k-tile g+NSTAGE-1 into the stage of k-tile g-1 (its readers
+//             finished before barrier g-1); wait until k-tile g+1 has landed; barrier g.
+//   consumer: k-steps 0..KS-2 of k-tile g (all LDS reads of its stage issued and complete);
+//             barrier g; last k-step, reading the first fragments of k-tile g+1 meanwhile.
+// The consumers issue no loads, so their stores (and bias loads) interfere with no counter; the
+// producers run ahead during an epilogue until the next barrier holds them.
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int SWZ, int NSTAGE, int OUTCLS, int PW>
+__global__ __launch_bounds__((WAVES_M * WAVES_N + PW) * 64) void gemm_mfma_ws_kernel(GemmParams p) {
+  constexpr int NWC = WAVES_M * WAVES_N;  // consumer waves
+  constexpr int NTP = PW * 64;            // producer threads
+  constexpr int CH = BK / 16;
+  constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int KS = BK / 32;
+  constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
+  constexpr int STAGE = A_BYTES + B_BYTES;
+  constexpr int STRIP = 32 * WTN, COLS = 4 * WTN;
+  constexpr int EPI_LDS = OUTCLS == OUT8 ? NWC * (STRIP + COLS) : 0;
+  constexpr int LDS_BYTES = NSTAGE * STAGE + EPI_LDS;
+  constexpr int DEPTH = NSTAGE - 1;
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % 64 == 0, "tile shape");
+  static_assert(NSTAGE >= 3 && LDS_BYTES <= 160 * 1024, "LDS budget");
+
+  __shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  // ---- this workgroup's items: ranks first, first + step, ... (count of them)
+  const int T = p.tiles_m * p.tiles_n;
+  const int W = T * p.batch;
+  int first, step, count;
+  {
+    const int G = (int)gridDim.x, b = (int)blockIdx.x;
+    if (G & 7) {
+      first = b;
+      step = G;
+      count = b < W ? (W - b + G - 1) / G : 0;
+    } else {
+      const int xcd = b & 7, l = b >> 3, nb = G >> 3;
+      const int per = W >> 3, rem = W & 7;
+      const int cnt = per + (xcd < rem ? 1 : 0);
+      first = xcd * per + min(xcd, rem) + l;
+      step = nb;
+      count = l < cnt ? (cnt - l + nb - 1) / nb : 0;
+    }
+    first = __builtin_amdgcn_readfirstlane(first);
+    step = __builtin_amdgcn_readfirstlane(step);
+    count = __builtin_amdgcn_readfirstlane(count);
+  }
+  if (count == 0) return;
+  auto locate = [&](int i, int& bz, int& m0, int& n0) {
+    const int g = first + i * step;
+    const int b_ = g / T;
+    int tm, tn;
+    tile_from_rank(p, g - b_ * T, tm, tn);
+    bz = __builtin_amdgcn_readfirstlane(b_);
+    m0 = __builtin_amdgcn_readfirstlane(tm * BM);
+    n0 = __builtin_amdgcn_readfirstlane(tn * BN);
+  };
+  const int KT = (p.K + BK - 1) / BK;
+  const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+
+  if (wave >= NWC) {
+    // ================================ producer ================================
+    const int ptid = tid - NWC * 64;
+    const int lda = (int)p.sAm, ldb = (int)p.sBn;
+    const unsigned wave_slot = __builtin_amdgcn_readfirstlane(lds_base + (wave - NWC) * 1024);
+    TileLoader<BM, BK, NTP, SWZ> la;
+    TileLoader<BN, BK, NTP, SWZ> lb;
+    la.init(ptid, 0, lda, p.K);
+    lb.init(ptid, 0, ldb, p.K);
+    constexpr int A_IT = decltype(la)::IT, B_IT = decltype(lb)::IT;
+    constexpr int LOADS = A_IT + B_IT;
+    static_assert(LOADS * DEPTH <= 63, "loads in flight must fit the counter");
+    const int OOB = (int)0x80000000;
+    v4i rA, rB;
+    int i_issue = 0, k_issue = 0, st_issue = 0, kt_left = 0;
+    auto aim = [&](int i) {
+      kt_left = KT;
+      k_issue = 0;
+      if (i < count) {
+        int bz, m0, n0;
+        locate(i, bz, m0, n0);
+        // rows at or past M (N) and bytes past K of the last row read as zero
+        rA = make_rsrc(p.A + (int64_t)bz * p.sAb + (int64_t)m0 * lda, (p.M - 1 - m0) * lda + p.K);
+        rB = make_rsrc(p.B + (int64_t)bz * p.sBb + (int64_t)n0 * ldb, (p.N - 1 - n0) * ldb + p.K);
+      } else {
+        // past the last item: empty buffers, zeros into stages nobody reads; the number of loads
+        // in flight, and so the count to wait for, stays constant
+        rA = make_rsrc(p.A, 0);
+        rB = make_rsrc(p.B, 0);
+      }
+    };
+    auto issue_ktile = [&]() {
+#pragma unroll
+      for (int d = 0; d < A_IT; ++d)
+        dma16_to_lds(rA, (k_issue < la.klim[d]) ? la.voff[d] : OOB, k_issue, wave_slot + st_issue * STAGE + d * NTP * 16);
+#pragma unroll
+      for (int d = 0; d < B_IT; ++d)
+        dma16_to_lds(rB, (k_issue < lb.klim[d]) ? lb.voff[d] : OOB, k_issue,
+                     wave_slot + st_issue * STAGE + A_BYTES + d * NTP * 16);
+      k_issue += BK;
+      st_issue = (st_issue + 1 == NSTAGE) ? 0 : st_issue + 1;
+      if (--kt_left == 0) {
+        ++i_issue;
+        aim(i_issue);
+      }
+    };
+    aim(0);
+#pragma unroll
+    for (int t = 0; t < DEPTH; ++t) issue_ktile();
+    wait_loads_and_barrier<LOADS*(DEPTH - 1)>();  // k-tile 0 landed
+    const int total = count * KT;
+    for (int g = 0; g < total; ++g) {
+      issue_ktile();                                // k-tile g + DEPTH
+      wait_loads_and_barrier<LOADS*(DEPTH - 1)>();  // k-tile g + 1 landed; barrier g
+    }
+    // the trailing (empty-buffer) loads still write zeros into LDS: they must land before the
+    // workgroup's LDS is handed to another one
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    return;
+  }
+
+  // ================================ consumer ================================
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  v16i acc[TM][TN];
+  const int frow = lane & 31;
+  const int fsw = (frow >> SWZ) & (CH - 1);
+  const int fhalf = lane >> 5;
+  const int a_lane = (wm * WTM + frow) * BK;
+  const int b_lane = A_BYTES + (wn * WTN + frow) * BK;
+  v4i fa[2][TM], fb[2][TN];
+  auto load_frag = [&](const char* stage, int ks, int buf, int r) {
+    const int coff = ((ks * 2 + fhalf) ^ fsw) * 16;
+    if (r < TM) fa[buf][r] = *(const v4i*)(stage + a_lane + r * 32 * BK + coff);
+    else fb[buf][r - TM] = *(const v4i*)(stage + b_lane + (r - TM) * 32 * BK + coff);
+  };
+  auto mfma = [&](int buf, int u) {
+    const int i = u / TN, j = u % TN;
+    if constexpr (OUTCLS == OUT8)  // rows of the MFMA result = n (4 consecutive n per lane)
+      acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
+    else  // rows of the MFMA result = m, lanes run along n
+      acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
+  };
+  constexpr int NM = TM * TN, NR = TM + TN;
+  // one k-step, pinned order: MFMA u, then fragment read u of the following k-step
+  auto kstep = [&](int buf, const char* rd_stage, int rd_ks) {
+#pragma unroll
+    for (int u = 0; u < NM; ++u) {
+      mfma(buf, u);
+#pragma unroll
+      for (int r = 0; r < NR; ++r)
+        if (NM > NR ? r == u : r * NM / NR == u) load_frag(rd_stage, rd_ks, buf ^ 1, r);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  const EpiCtx e = make_epi(p);
+
+  asm volatile("s_barrier" ::: "memory");  // k-tile 0 is in LDS
+  int st = 0;
+  for (int it = 0; it < count; ++it) {
+    int bz, m0, n0;
+    locate(it, bz, m0, n0);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+#pragma unroll
+    for (int r = 0; r < NR; ++r) load_frag(lds + st * STAGE, 0, 0, r);
+    for (int kt = 0; kt < KT; ++kt) {
+      const char* cur = lds + st * STAGE;
+      st = (st + 1 == NSTAGE) ? 0 : st + 1;
+#pragma unroll
+      for (int ks = 0; ks < KS - 1; ++ks) kstep(ks & 1, cur, ks + 1);
+      // every LDS read of this k-tile is issued: wait for them, then hand the stage back
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      // last k-step; the fragments it fetches are the first of the next k-tile (of the next item
+      // after the last k-tile: landed as well, and simply fetched again at the item's start)
+      kstep((KS - 1) & 1, lds + st * STAGE, 0);
+    }
+    stream_epilogue<TM, TN, OUTCLS>(p, e, acc, bz, m0 + wm * WTM, n0 + wn * WTN,
+                                    lds + NSTAGE * STAGE + wave * (STRIP + COLS), lane);
+  }
 }
 
 // ---- gather family -----------------------------------------------------------------------------
@@ -1122,6 +1337,15 @@ struct Config {
         BM, BN, BK, WM * WN * 64, true, false, OCC                                        \
   }
 
+#define TI_WS(BM, BN, BK, WM, WN, SWZ, NS, PW)                                            \
+  {                                                                                       \
+    "ws_" #BM "x" #BN "x" #BK "_w" #WM "x" #WN "_s" #SWZ "_p" #NS "_l" #PW,                 \
+        {gemm_mfma_ws_kernel<BM, BN, BK, WM, WN, SWZ, NS, OUT8, PW>,                        \
+         gemm_mfma_ws_kernel<BM, BN, BK, WM, WN, SWZ, NS, OUT32, PW>,                       \
+         gemm_mfma_ws_kernel<BM, BN, BK, WM, WN, SWZ, NS, OUT16, PW>},                      \
+        BM, BN, BK, (WM * WN + PW) * 64, true, false, 1                                   \
+  }
+
 enum ConfigId {
   CFG_GATHER = 0,
   CFG_TILE_256x128,   // one tile per workgroup: any output layout the fast loads allow
@@ -1132,8 +1356,7 @@ enum ConfigId {
   CFG_SKINNY_32,
   CFG_SKINNY_64,
   CFG_STREAM_256x256,       // persistent: row-major, 16-byte aligned outputs
-  CFG_STREAM_256x256_WIDE,  // waves 128 columns wide: int8 rows leave as whole 128-byte lines
-  CFG_STREAM_256x128,
+  CFG_WS_256x128,           // persistent, loads issued by dedicated producer waves
   CFG_STREAM_128x128,
 };
 
@@ -1147,8 +1370,7 @@ static const Config g_configs[] = {
     {"skinny_m32_slab16", {gemm_skinny_kernel<OUT8, 2>, gemm_skinny_kernel<OUT32, 2>, gemm_skinny_kernel<OUT16, 2>}, 32, 16, 64, 512, true, true},
     {"skinny_m64_slab16", {gemm_skinny_kernel<OUT8, 4>, gemm_skinny_kernel<OUT32, 4>, gemm_skinny_kernel<OUT16, 4>}, 64, 16, 64, 512, true, true},
     TI_STREAM(256, 256, 64, 2, 4, 2, 4, 1),
-    TI_STREAM(256, 256, 64, 4, 2, 2, 3, 1),
-    TI_STREAM(256, 128, 128, 2, 2, 1, 3, 1),
+    TI_WS(256, 128, 128, 2, 2, 1, 3, 4),
     TI_STREAM(128, 128, 64, 2, 2, 2, 3, 2),
 };
 static const int g_num_configs = (int)(sizeof(g_configs) / sizeof(g_configs[0]));
@@ -1191,18 +1413,20 @@ static bool stream_eligible(const GemmParams& p) {
 
 // Tile choice: score = (measured relative efficiency of the tile class) x (fraction of the
 // 256 CUs kept busy over all rounds of workgroups) x (fraction of the tiles' area that is real
-// output).  The class efficiencies were measured with weights streamed from HBM.  Outputs the
-// persistent kernels can store (row-major, aligned) go to them; the rest to the one-tile kernels.
+// output) x (a small bonus for few rounds: a chip that is partly idle in its only round runs
+// that round faster than a full chip runs the first of two).  The class efficiencies were measured
+// with weights streamed from HBM.  Outputs the persistent kernels can store (row-major, aligned)
+// go to them; the rest to the one-tile kernels.
 static int pick_config(const GemmParams& p) {
   if (!fast_eligible(p)) return CFG_GATHER;
   if (p.M <= 64) return CFG_SKINNY_16 + (p.M > 16) + (p.M > 32);
   const bool stream = stream_eligible(p);
-  // short K, int8 out: the epilogue and its stores dominate, whole-line stores pay
-  const bool wide = out_class(p.out_dtype) == OUT8 && p.K <= 256;
+  // short K: the epilogue dominates and the larger tile halves the operand traffic per output
+  const double big = p.K <= 512 ? 1.20 : 0.97;
   struct Cand { int cfg; double base; };
   const Cand cands[] = {
-      {stream ? (wide ? CFG_STREAM_256x256_WIDE : CFG_STREAM_256x256) : CFG_TILE_256x256, 1.00},
-      {stream ? CFG_STREAM_256x128 : CFG_TILE_256x128, 0.90},
+      {stream ? CFG_STREAM_256x256 : CFG_TILE_256x256, stream ? big : 1.00},
+      {stream ? CFG_WS_256x128 : CFG_TILE_256x128, stream ? 1.00 : 0.90},
       {stream ? CFG_STREAM_128x128 : CFG_TILE_128x128, 0.78},
       {CFG_TILE_64x64, 0.50},
   };
@@ -1216,7 +1440,7 @@ static int pick_config(const GemmParams& p) {
     const int64_t rounds = (tiles + slots - 1) / slots;
     const double busy = (double)tiles / (double)(rounds * slots);
     const double area = ((double)p.M * p.N) / ((double)(tm * k.bm) * (double)(tn * k.bn));
-    const double score = c.base * busy * area;
+    const double score = c.base * busy * area * (1.0 + 0.1 / (double)rounds);
     if (score > best_score) best_score = score, best = c.cfg;
   }
   return best;
