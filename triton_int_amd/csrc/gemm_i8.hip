@@ -1030,10 +1030,29 @@ __global__ __launch_bounds__((WAVES_M * WAVES_N + PW) * 64) void gemm_mfma_ws_ke
     for (int t = 0; t < DEPTH; ++t) issue_ktile();
     wait_loads_and_barrier<LOADS*(DEPTH - 1)>();  // k-tile 0 landed
     const int total = count * KT;
+#ifdef TI_TRACE
+    uint64_t tr_issue = 0, tr_wait = 0, tr_bar = 0;
+    const uint64_t tr_w0 = wall_clock64();
+    for (int g = 0; g < total; ++g) {
+      const uint64_t c0 = __builtin_readcyclecounter();
+      issue_ktile();
+      const uint64_t c1 = __builtin_readcyclecounter();
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS*(DEPTH - 1)) : "memory");
+      const uint64_t c2 = __builtin_readcyclecounter();
+      asm volatile("s_barrier" ::: "memory");
+      const uint64_t c3 = __builtin_readcyclecounter();
+      tr_issue += c1 - c0; tr_wait += c2 - c1; tr_bar += c3 - c2;
+    }
+    if (lane == 0 && blockIdx.x < 256) {
+      unsigned long long* tr = ti_trace_buf + (blockIdx.x * 4 + (wave & 3)) * 8;
+      tr[0] = tr_issue; tr[1] = tr_wait; tr[2] = tr_bar; tr[3] = total; tr[4] = wall_clock64() - tr_w0;
+    }
+#else
     for (int g = 0; g < total; ++g) {
       issue_ktile();                                // k-tile g + DEPTH
       wait_loads_and_barrier<LOADS*(DEPTH - 1)>();  // k-tile g + 1 landed; barrier g
     }
+#endif
     // the trailing (empty-buffer) loads still write zeros into LDS: they must land before the
     // workgroup's LDS is handed to another one
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");

@@ -57,84 +57,111 @@ __device__ __forceinline__ float norm_one(float x, float mean, float rstd, float
   return has_b ? o + b : o;
 }
 
+// Persistent: a workgroup walks rows blockIdx.x, blockIdx.x + gridDim.x, ...  gamma and beta are
+// row-invariant and stay in registers for all of them (re-reading them per row would triple the
+// bytes that cross the L2 -> CU path), and for the plain LayerNorm the next row's loads are issued
+// before the current row's reductions so that they are in flight during the two block-wide sums.
 template <int VPT, bool DQ>
 __global__ __launch_bounds__(RN_THREADS) void rownorm_vec_kernel(RowNormParams p) {
   __shared__ float red[RN_WAVES];
   const int tid = threadIdx.x;
-  const int row = blockIdx.x;
   const int nvec = p.cols >> 2;
+  const bool has_b = p.beta != nullptr;
+  const v4f zero4 = {0.f, 0.f, 0.f, 0.f};
 
-  v4f x[VPT];
+  v4f w[VPT], b[VPT];
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
     const int v = tid + j * RN_THREADS;
-    if (v < nvec) {
-      if constexpr (DQ) {
-        // streamed once: non-temporal, so the rows do not displace gamma/beta in the caches
-        const v4i a = __builtin_nontemporal_load((const v4i*)(p.acc + (int64_t)row * p.acc_rs + v * 4));
-        const v4f r = __builtin_nontemporal_load((const v4f*)(p.resid_in + (int64_t)row * p.rin_rs + v * 4));
-        v4f o;
+    w[j] = v < nvec ? *(const v4f*)(p.gamma + v * 4) : zero4;
+    b[j] = (has_b && v < nvec) ? *(const v4f*)(p.beta + v * 4) : zero4;
+  }
+
+  auto load_x = [&](int row, v4f (&dst)[VPT]) {
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          // functional/fused.py:9: residual + alpha * int32 (product and sum rounded separately)
-          const float prod = p.in_scale * (float)a[t];
-          o[t] = r[t] + prod;
+    for (int j = 0; j < VPT; ++j) {
+      const int v = tid + j * RN_THREADS;
+      // streamed once: non-temporal
+      dst[j] = v < nvec ? __builtin_nontemporal_load((const v4f*)(p.x + (int64_t)row * p.x_rs + v * 4)) : zero4;
+    }
+  };
+
+  v4f x[VPT], xn[VPT];
+  int row = blockIdx.x;
+  if constexpr (!DQ) {
+    if (row < p.rows) load_x(row, xn);
+  }
+  const float inv_n = 1.0f / (float)p.cols;
+  const bool y_vec = p.y && ((p.y_rs & 3) == 0) && ((((uintptr_t)p.y) & 3) == 0);
+
+  for (; row < p.rows; row += gridDim.x) {
+    if constexpr (DQ) {
+#pragma unroll
+      for (int j = 0; j < VPT; ++j) {
+        const int v = tid + j * RN_THREADS;
+        if (v < nvec) {
+          const v4i a = __builtin_nontemporal_load((const v4i*)(p.acc + (int64_t)row * p.acc_rs + v * 4));
+          const v4f r = __builtin_nontemporal_load((const v4f*)(p.resid_in + (int64_t)row * p.rin_rs + v * 4));
+          v4f o;
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            // functional/fused.py:9: residual + alpha * int32 (product and sum rounded separately)
+            const float prod = p.in_scale * (float)a[t];
+            o[t] = r[t] + prod;
+          }
+          x[j] = o;
+          __builtin_nontemporal_store(o, (v4f*)(p.resid_out + (int64_t)row * p.rout_rs + v * 4));
+        } else {
+          x[j] = zero4;
         }
-        x[j] = o;
-        __builtin_nontemporal_store(o, (v4f*)(p.resid_out + (int64_t)row * p.rout_rs + v * 4));
-      } else {
-        x[j] = __builtin_nontemporal_load((const v4f*)(p.x + (int64_t)row * p.x_rs + v * 4));
       }
     } else {
-      x[j] = (v4f){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < VPT; ++j) x[j] = xn[j];
+      const int next = row + (int)gridDim.x;
+      if (next < p.rows) load_x(next, xn);
     }
-  }
 
-  const float inv_n = 1.0f / (float)p.cols;
-  float mean = 0.0f;
-  if (!p.rms) {
-    float s = 0.0f;
+    float mean = 0.0f;
+    if (!p.rms) {
+      float s = 0.0f;
 #pragma unroll
-    for (int j = 0; j < VPT; ++j) s += (x[j][0] + x[j][1]) + (x[j][2] + x[j][3]);
-    mean = block_sum(s, red, tid) * inv_n;
-  }
-  float m2 = 0.0f;
-#pragma unroll
-  for (int j = 0; j < VPT; ++j) {
-    const int v = tid + j * RN_THREADS;
-    if (v < nvec) {
-      const float d0 = x[j][0] - mean, d1 = x[j][1] - mean, d2 = x[j][2] - mean, d3 = x[j][3] - mean;
-      m2 += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
+      for (int j = 0; j < VPT; ++j) s += (x[j][0] + x[j][1]) + (x[j][2] + x[j][3]);
+      mean = block_sum(s, red, tid) * inv_n;
     }
-  }
-  const float var = block_sum(m2, red, tid) * inv_n;
-  const float rstd = 1.0f / sqrtf(var + p.eps);
-  if (tid == 0) {
-    if (p.mean_out) p.mean_out[row] = mean;
-    if (p.rstd_out) p.rstd_out[row] = rstd;
-  }
+    float m2 = 0.0f;
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) {
+      const int v = tid + j * RN_THREADS;
+      if (v < nvec) {
+        const float d0 = x[j][0] - mean, d1 = x[j][1] - mean, d2 = x[j][2] - mean, d3 = x[j][3] - mean;
+        m2 += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
+      }
+    }
+    const float var = block_sum(m2, red, tid) * inv_n;
+    const float rstd = 1.0f / sqrtf(var + p.eps);
+    if (tid == 0) {
+      if (p.mean_out) p.mean_out[row] = mean;
+      if (p.rstd_out) p.rstd_out[row] = rstd;
+    }
 
-  const bool has_b = p.beta != nullptr;
-  const bool y_vec = p.y && ((p.y_rs & 3) == 0) && ((((uintptr_t)p.y) & 3) == 0);
 #pragma unroll
-  for (int j = 0; j < VPT; ++j) {
-    const int v = tid + j * RN_THREADS;
-    if (v < nvec) {
-      const v4f w = *(const v4f*)(p.gamma + v * 4);
-      v4f b = {0.f, 0.f, 0.f, 0.f};
-      if (has_b) b = *(const v4f*)(p.beta + v * 4);
-      v4f o;
+    for (int j = 0; j < VPT; ++j) {
+      const int v = tid + j * RN_THREADS;
+      if (v < nvec) {
+        v4f o;
 #pragma unroll
-      for (int t = 0; t < 4; ++t) o[t] = norm_one(x[j][t], mean, rstd, w[t], b[t], has_b);
-      if (p.ln_out) __builtin_nontemporal_store(o, (v4f*)(p.ln_out + (int64_t)row * p.ln_rs + v * 4));
-      if (p.y) {
-        const int q0 = q8(o[0], p.round_mode), q1 = q8(o[1], p.round_mode), q2 = q8(o[2], p.round_mode),
-                  q3 = q8(o[3], p.round_mode);
-        int8_t* dst = p.y + (int64_t)row * p.y_rs + v * 4;
-        if (y_vec) {
-          __builtin_nontemporal_store(pack4(q0, q1, q2, q3), (unsigned*)dst);
-        } else {
-          dst[0] = (int8_t)q0; dst[1] = (int8_t)q1; dst[2] = (int8_t)q2; dst[3] = (int8_t)q3;
+        for (int t = 0; t < 4; ++t) o[t] = norm_one(x[j][t], mean, rstd, w[j][t], b[j][t], has_b);
+        if (p.ln_out) __builtin_nontemporal_store(o, (v4f*)(p.ln_out + (int64_t)row * p.ln_rs + v * 4));
+        if (p.y) {
+          const int q0 = q8(o[0], p.round_mode), q1 = q8(o[1], p.round_mode), q2 = q8(o[2], p.round_mode),
+                    q3 = q8(o[3], p.round_mode);
+          int8_t* dst = p.y + (int64_t)row * p.y_rs + v * 4;
+          if (y_vec) {
+            __builtin_nontemporal_store(pack4(q0, q1, q2, q3), (unsigned*)dst);
+          } else {
+            dst[0] = (int8_t)q0; dst[1] = (int8_t)q1; dst[2] = (int8_t)q2; dst[3] = (int8_t)q3;
+          }
         }
       }
     }
@@ -207,6 +234,9 @@ static int launch_rownorm(const RowNormParams& p, hipStream_t stream) {
     return launch_status("rownorm_any_kernel");
   }
   const int vpt = (p.cols / 4 + RN_THREADS - 1) / RN_THREADS;
+  // persistent workgroups: a few per CU, each walking several rows
+  const unsigned slots = 256u * (vpt <= 2 ? 8u : (vpt <= 5 ? 4u : 3u));
+  if (grid.x > slots) grid.x = slots;
   if (vpt <= 1) rownorm_vec_kernel<1, DQ><<<grid, block, 0, stream>>>(p);
   else if (vpt <= 2) rownorm_vec_kernel<2, DQ><<<grid, block, 0, stream>>>(p);
   else if (vpt <= 3) rownorm_vec_kernel<3, DQ><<<grid, block, 0, stream>>>(p);
