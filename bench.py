@@ -23,6 +23,12 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 METRIC = "int8 GEMM TOPS (% MFMA peak), LN/GELU GB/s, W8A8 OPT-13B layer ms"
+# Bytes that crossed the L2 <-> fabric boundary per launch of a kernel on this workload (average over
+# the launches of one step), from rocprofv3 FETCH_SIZE and WRITE_SIZE passes scaled by the same
+# counters' readings for a 256 MiB device copy (x2.0 and x1.0); see profiles/.
+MEASURED_TRAFFIC_BYTES = {
+    "ws_256x128x128_w2x2_s1_p3_l4/int8": (2.0 * 52601 + 1.0 * 15384) * 1024,
+}
 INT8_PEAK_TOPS = 5000.0   # MI355X dense INT8 MFMA, published
 HBM_PEAK_GBPS = 8000.0    # MI355X HBM3E, published
 
@@ -116,6 +122,59 @@ def mfma_issue_peak(torch, lib, random_operands):
     torch.cuda.synchronize()
     assert rc == 0
     return ops.value / (s.elapsed_time(e) * 1e-3) / 1e12
+
+
+def sustained_clock(torch, dev, seconds=2.5):
+    """fc2-shaped GEMM (2048 x 4096 x 16384, fp32 out) looped for `seconds` while rocm-smi is sampled
+    from a thread: sustained TOPS and the shader clock the chip holds under that load, once with
+    uniform random int8 operands and once with all-zero operands (same instruction stream, no
+    operand toggling).  The difference is the power limit, not the kernel."""
+    import re
+    import subprocess
+    import threading
+
+    from triton_int_amd.kernels import linear
+
+    M, N, K = 2048, 4096, 16384
+    out = {}
+    for kind in ("uniform", "zeros"):
+        if kind == "uniform":
+            ws = [torch.randint(-127, 128, (N, K), dtype=torch.int8, device=dev) for _ in range(8)]
+            x = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=dev)
+        else:
+            ws = [torch.zeros((N, K), dtype=torch.int8, device=dev) for _ in range(8)]
+            x = torch.zeros((M, K), dtype=torch.int8, device=dev)
+        y = torch.empty((M, N), dtype=torch.float32, device=dev)
+        clocks = []
+
+        def sample():
+            for _ in range(int(seconds / 0.5)):
+                time.sleep(0.4)
+                try:
+                    r = subprocess.run(["/opt/rocm/bin/rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=5)
+                    m = re.search(r"sclk clock level:[^(]*\((\d+)Mhz\)", r.stdout)
+                    if m:
+                        clocks.append(int(m.group(1)))
+                except Exception:
+                    pass
+
+        th = threading.Thread(target=sample)
+        th.start()
+        t0, n = time.perf_counter(), 0
+        while time.perf_counter() - t0 < seconds:
+            for i in range(50):
+                linear.linear_a8_w8_ofp32(x, ws[i % 8], 0.002, out=y)
+            torch.cuda.synchronize()
+            n += 50
+        el = time.perf_counter() - t0
+        th.join()
+        out[kind] = {"TOPS": 2.0 * M * N * K * n / el / 1e12, "us_per_gemm": el / n * 1e6,
+                     "sclk_mhz": (sorted(clocks)[len(clocks) // 2] if clocks else None)}
+        if out[kind]["sclk_mhz"]:
+            # MFMA peak at the clock actually held: 256 CUs x 8192 int8 ops per clock
+            out[kind]["frac_of_peak_at_held_clock"] = out[kind]["TOPS"] * 1e12 / (256 * 8192 * out[kind]["sclk_mhz"] * 1e6)
+        del ws, x, y
+    return out
 
 
 def extras(torch, dev):
@@ -213,6 +272,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU emulation baseline")
     ap.add_argument("--no-extra", action="store_true", help="skip the row-kernel / BMM extras")
+    ap.add_argument("--calib-copy-mb", type=int, default=0,
+                    help="before the timed region, run 4 device-to-device copies of this many MiB: a kernel of "
+                         "known traffic to scale rocprofv3's FETCH_SIZE / WRITE_SIZE readings with")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (every op shards over "
@@ -251,6 +313,14 @@ def main():
             m(x)
             if ev is not None and i == n_dom - 1:
                 ev[1].record()
+
+    if args.calib_copy_mb > 0:
+        src = torch.randint(-127, 128, (args.calib_copy_mb << 20,), dtype=torch.int8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step()
@@ -293,7 +363,9 @@ def main():
             "peak": INT8_PEAK_TOPS,
             "unit": "TFLOP/s",
             "frac": achieved / INT8_PEAK_TOPS,
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(dominant),
+            "algorithmic_bytes": sum(x.numel() + m.weight.numel() + x.shape[0] * m.weight.shape[0]
+                                     for _, m, x, _ in groups[dominant]) / n_dom,
             "launches_per_step": n_dom,
             "avg_launch_us": dom_ms * 1e3 / n_dom,
             "ops_per_launch": dom_ops / n_dom,
@@ -307,6 +379,7 @@ def main():
     if not args.no_extra:
         result["extra"] = extras(torch, dev)
         result["extra"]["opt13b_decoder_layer"] = decoder_layer_ms(torch, dev)
+        result["extra"]["sustained_fc2_2048x4096x16384"] = sustained_clock(torch, dev)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch, layers)
     print(json.dumps(result))

@@ -1466,9 +1466,11 @@ static int pick_config(const GemmParams& p) {
 }
 
 static int pick_group_m(const GemmParams& p, const Config& k) {
-  // each XCD runs tiles/8 consecutive tiles; make that range roughly square in rows touched
+  // Each XCD is dealt tiles/8 consecutive tiles and has 32 CUs: the tiles it runs at the same
+  // time share its L2, so that set should touch as few operand rows as possible (roughly square).
   const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
-  const int per_xcd = (int)((tiles + 7) / 8);
+  const int at_once = 32 * (k.stream_occ > 1 ? k.stream_occ : 1);
+  const int per_xcd = (int)((tiles + 7) / 8) < at_once ? (int)((tiles + 7) / 8) : at_once;
   int best = 1;
   int64_t best_cost = -1;
   for (int g = 1; g <= p.tiles_m && g <= 64; g *= 2) {
