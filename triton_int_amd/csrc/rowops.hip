@@ -262,6 +262,11 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// Per element the work is: byte -> float (v_cvt_f32_ubyteN on the sign-flipped dword, so the float
+// is x + 128), one fma that forms (x - max) * scale * log2(e), the hardware exp2, one add for the
+// sum; then one fma e * (127 / sum) + 1.5 * 2^23, whose low byte is the rounded probability (it
+// lies in [0, 127], no clamp), and byte permutes to pack.  16-byte chunks that lie wholly beyond a
+// causal limit are neither read nor computed, the one chunk that straddles it is masked.
 template <int VPT>
 __global__ __launch_bounds__(SM_WAVES * 64) void softmax_q_kernel(const int8_t* __restrict__ x, int64_t x_rs,
                                                                   float scale, int8_t* __restrict__ y, int64_t y_rs,
@@ -273,35 +278,59 @@ __global__ __launch_bounds__(SM_WAVES * 64) void softmax_q_kernel(const int8_t* 
   const int8_t* xr = x + (int64_t)row * x_rs;
   int8_t* yr = y + (int64_t)row * y_rs;
   const bool vec = ((((uintptr_t)xr) | ((uintptr_t)yr)) & 15) == 0;
+  const float NEG = -1.0f;  // below every x + 128 >= 0: excluded from the maximum, flags a masked element
 
-  int v[VPT][16];
-  int mx = -128;
+  // f[j][t] = x + 128 as a float, or NEG for masked / out-of-row elements
+  float f[VPT][16];
+  float mx = NEG;
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
     const int c0 = (j * 64 + lane) * 16;
-    if (vec && c0 + 16 <= cols) {
-      const v4i w = __builtin_nontemporal_load((const v4i*)(xr + c0));
+    if (c0 >= limit) {
 #pragma unroll
-      for (int t = 0; t < 16; ++t) v[j][t] = (int)(int8_t)(w[t >> 2] >> ((t & 3) * 8));
+      for (int t = 0; t < 16; ++t) f[j][t] = NEG;
+    } else if (vec && c0 + 16 <= limit) {
+      v4u w = __builtin_nontemporal_load((const v4u*)(xr + c0));
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const unsigned u = w[g] ^ 0x80808080u;
+        // the compiler turns these into v_cvt_f32_ubyte0..3
+        f[j][4 * g + 0] = (float)(u & 0xffu);
+        f[j][4 * g + 1] = (float)((u >> 8) & 0xffu);
+        f[j][4 * g + 2] = (float)((u >> 16) & 0xffu);
+        f[j][4 * g + 3] = (float)(u >> 24);
+      }
+#pragma unroll
+      for (int t = 0; t < 16; t += 2) mx = fmaxf(fmaxf(mx, f[j][t]), f[j][t + 1]);  // v_max3_f32
     } else {
 #pragma unroll
-      for (int t = 0; t < 16; ++t) v[j][t] = c0 + t < cols ? (int)xr[c0 + t] : -128;
+      for (int t = 0; t < 16; ++t) {
+        f[j][t] = c0 + t < limit ? (float)((int)xr[c0 + t] + 128) : NEG;
+        mx = fmaxf(mx, f[j][t]);
+      }
     }
-#pragma unroll
-    for (int t = 0; t < 16; ++t)
-      if (c0 + t < limit) mx = max(mx, v[j][t]);
   }
-  mx = (int)wave_max((float)mx);  // |x| <= 128: exact in fp32
-  float e[VPT][16];
+  mx = wave_max(mx);
+  const float s2 = scale * 1.44269504088896340736f;  // exp(v) = exp2(v * log2 e)
+  const float c = -(mx * s2);
   float sum = 0.0f;
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
     const int c0 = (j * 64 + lane) * 16;
+    if (c0 >= limit) continue;
+    if (c0 + 16 <= limit) {
 #pragma unroll
-    for (int t = 0; t < 16; ++t) {
-      const float ex = __expf((float)(v[j][t] - mx) * scale);
-      e[j][t] = c0 + t < limit ? ex : 0.0f;
-      sum += e[j][t];
+      for (int t = 0; t < 16; ++t) {
+        f[j][t] = __builtin_amdgcn_exp2f(__builtin_fmaf(f[j][t], s2, c));
+        sum += f[j][t];
+      }
+    } else {  // the chunk that straddles the limit (or the end of the row)
+#pragma unroll
+      for (int t = 0; t < 16; ++t) {
+        const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(f[j][t], s2, c));
+        f[j][t] = f[j][t] < 0.0f ? 0.0f : e;
+        sum += f[j][t];
+      }
     }
   }
   sum = wave_sum(sum);
@@ -309,13 +338,20 @@ __global__ __launch_bounds__(SM_WAVES * 64) void softmax_q_kernel(const int8_t* 
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
     const int c0 = (j * 64 + lane) * 16;
-    unsigned w[4];
+    if (c0 >= cols) continue;
+    v4u w = {0u, 0u, 0u, 0u};
+    if (c0 < limit) {
 #pragma unroll
-    for (int g = 0; g < 4; ++g)
-      w[g] = pack4(q8<false>(e[j][4 * g] * r), q8<false>(e[j][4 * g + 1] * r), q8<false>(e[j][4 * g + 2] * r),
-                   q8<false>(e[j][4 * g + 3] * r));
+      for (int g = 0; g < 4; ++g) {
+        const unsigned b0 = __float_as_uint(__builtin_fmaf(f[j][4 * g + 0], r, 12582912.0f));
+        const unsigned b1 = __float_as_uint(__builtin_fmaf(f[j][4 * g + 1], r, 12582912.0f));
+        const unsigned b2 = __float_as_uint(__builtin_fmaf(f[j][4 * g + 2], r, 12582912.0f));
+        const unsigned b3 = __float_as_uint(__builtin_fmaf(f[j][4 * g + 3], r, 12582912.0f));
+        w[g] = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u) | __builtin_amdgcn_perm(b3, b2, 0x04000c0cu);
+      }
+    }
     if (vec && c0 + 16 <= cols) {
-      __builtin_nontemporal_store((v4u){w[0], w[1], w[2], w[3]}, (v4u*)(yr + c0));
+      __builtin_nontemporal_store(w, (v4u*)(yr + c0));
     } else {
 #pragma unroll
       for (int t = 0; t < 16; ++t)
