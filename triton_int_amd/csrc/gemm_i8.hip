@@ -1198,50 +1198,73 @@ __global__ __launch_bounds__(256) void gemm_gather_kernel(GemmParams p) {
 // The 8 waves of a workgroup either take 8 different slabs (short K) or split K between them
 // (each a contiguous run of k-steps, so a wave reads whole cache lines) and add their
 // int32 partial sums through LDS — integer addition, so the result does not depend on the split.
-template <int OUTCLS, int MBMAX>
-__global__ __launch_bounds__(512) void gemm_skinny_kernel(GemmParams p) {
+template <int OUTCLS, int MBMAX, int G = 1, int UU = 0>
+__global__ __launch_bounds__(512, UU ? 2 : 4) void gemm_skinny_kernel(GemmParams p) {
   constexpr int NW = 8;
-  constexpr int U = 8 / MBMAX;  // k-steps per batch of loads; two batches are in flight
-  __shared__ int red[NW][MBMAX][256];
+  constexpr int U = UU ? UU : (MBMAX * G == 1 ? 6 : 8 / (MBMAX * G));  // k-steps per batch of loads; two batches are in flight
+  __shared__ int red[NW][G * MBMAX][256];
   const int tid = threadIdx.x, lane = tid & 63;
+#ifdef TI_TRACE
+  const uint64_t tr0 = wall_clock64();
+#endif
   // The wave index must be known to be wave-uniform: the trip counts below depend on it, and a
   // branch the compiler believes divergent would wrap MFMAs in EXEC masking, which MFMAs ignore.
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ksplit = p.ksplit;
-  const int slab = blockIdx.x * (NW / ksplit) + wave / ksplit;
+  // a wave owns a group of G consecutive 16-row slabs of B (they share the A fragments it loads)
+  // and one of the ksplit contiguous runs of K
+  const int group = blockIdx.x * (NW / ksplit) + wave / ksplit;
   const int kpart = wave % ksplit;
   const int bz = blockIdx.y;
   const int MB = (p.M + 15) >> 4;
   const int r16 = lane & 15, c4 = lane >> 4;
   const int8_t* Ab = p.A + (int64_t)bz * p.sAb;
   const int8_t* Bb = p.B + (int64_t)bz * p.sBb;
-  const int n_row = min(slab * 16 + r16, p.N - 1);
-  const int8_t* wrow = Bb + (int64_t)n_row * p.sBn + c4 * 16;
+  const int8_t* wrow[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) wrow[g] = Bb + (int64_t)min((group * G + g) * 16 + r16, p.N - 1) * p.sBn + c4 * 16;
   const int8_t* xrow[MBMAX];
 #pragma unroll
   for (int mb = 0; mb < MBMAX; ++mb) xrow[mb] = Ab + (int64_t)min(mb * 16 + r16, p.M - 1) * p.sAm + c4 * 16;
 
-  v4i acc[MBMAX];
+  v4i acc[G][MBMAX];
 #pragma unroll
-  for (int mb = 0; mb < MBMAX; ++mb) acc[mb] = (v4i){0, 0, 0, 0};
+  for (int g = 0; g < G; ++g)
+#pragma unroll
+    for (int mb = 0; mb < MBMAX; ++mb) acc[g][mb] = (v4i){0, 0, 0, 0};
 
-  // Whole 64-byte k-steps of this wave's run go in batches of U
-  // with two register sets: the loads of batch b+1 are issued before the MFMAs of batch b, so a
-  // wave keeps up to 2*U weight loads (1 KB each) in flight, and nothing in the batch loop looks
-  // at a loaded value before the MFMAs do.  Left-over k-steps and a K tail (K % 64 != 0, the only
-  // place that needs zero fill) are handled one at a time afterwards.  The weight stream bypasses
-  // the caches (non-temporal); A is re-read by every slab and is served by L2.
+  // The epilogue's scalars and per-column terms are fetched now, ahead of the weight stream: at the
+  // end of the kernel each of them would cost a full memory round trip with nothing to overlap.
+  const EpiCtx e = make_epi(p);
+  float col[G][4];
+  int bias_i32[G][4];
+#pragma unroll
+  for (int g = 0; g < G; ++g)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int n = min((group * G + g) * 16 + 4 * c4 + i, p.N - 1);
+      col[g][i] = column_term(e, n);
+      bias_i32[g][i] = (e.epilogue == TI_EPI_I32 && e.bias_kind == TI_BIAS_I32) ? ((const int*)e.bias)[n] : 0;
+    }
+
+  // Whole 64-byte k-steps of this wave's run go in batches of U with two register sets: the loads
+  // of batch b+1 are issued before the MFMAs of batch b, so a wave keeps up to 2*U*G weight loads
+  // (1 KB each) in flight, and nothing in the batch loop looks at a loaded value before the MFMAs
+  // do.  Left-over k-steps and a K tail (K % 64 != 0, the only place that needs zero fill) are
+  // handled one at a time afterwards.  A is re-read by every group and is served by L2.
   const int KSF = p.K >> 6;  // whole k-steps
   const int per = (KSF + ksplit - 1) / ksplit;  // each wave takes a contiguous run of k-steps
   const int j0 = kpart * per;
   const int nj = min(max(KSF - j0, 0), per);
   const int nb = nj / U;
   constexpr int kstride = 64;
-  v4i wf[2][U], xf[2][U][MBMAX];
+  v4i wf[2][U][G], xf[2][U][MBMAX];
   auto load_batch = [&](int buf, int b) {
     const int k0 = (j0 + b * U) * 64;
 #pragma unroll
-    for (int u = 0; u < U; ++u) wf[buf][u] = *(const v4i*)(wrow + k0 + u * kstride);
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int g = 0; g < G; ++g) wf[buf][u][g] = *(const v4i*)(wrow[g] + k0 + u * kstride);
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -1251,8 +1274,10 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(GemmParams p) {
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int mb = 0; mb < MBMAX; ++mb)
-        acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[buf][u], xf[buf][u][mb], acc[mb], 0, 0, 0);
+      for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int mb = 0; mb < MBMAX; ++mb)
+          acc[g][mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[buf][u][g], xf[buf][u][mb], acc[g][mb], 0, 0, 0);
   };
   if (nb > 0) load_batch(0, 0);
   for (int b = 0; b < nb; b += 2) {
@@ -1262,67 +1287,82 @@ __global__ __launch_bounds__(512) void gemm_skinny_kernel(GemmParams p) {
     if (b + 2 < nb) load_batch(0, b + 2);
     compute(1);
   }
-  // left-over whole k-steps (fewer than U): one more batch, loads first, guarded by wave-uniform tests
-  const int rem = nj - nb * U;
-  if (rem > 0) {
-    const int k0 = (j0 + nb * U) * 64;
+  // left-over whole k-steps (fewer than U), then the K tail: one k-step at a time
+  for (int j = nb * U; j < nj; ++j) {
+    const int k0 = (j0 + j) * 64;
+    v4i w1[G], x1[MBMAX];
 #pragma unroll
-    for (int u = 0; u < U - 1; ++u)
-      if (u < rem) wf[0][u] = *(const v4i*)(wrow + k0 + u * kstride);
+    for (int g = 0; g < G; ++g) w1[g] = *(const v4i*)(wrow[g] + k0);
 #pragma unroll
-    for (int u = 0; u < U - 1; ++u)
-      if (u < rem) {
+    for (int mb = 0; mb < MBMAX; ++mb) x1[mb] = *(const v4i*)(xrow[mb] + k0);
 #pragma unroll
-        for (int mb = 0; mb < MBMAX; ++mb) xf[0][u][mb] = *(const v4i*)(xrow[mb] + k0 + u * kstride);
-      }
+    for (int g = 0; g < G; ++g)
 #pragma unroll
-    for (int u = 0; u < U - 1; ++u)
-      if (u < rem) {
-#pragma unroll
-        for (int mb = 0; mb < MBMAX; ++mb)
-          acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[0][u], xf[0][u][mb], acc[mb], 0, 0, 0);
-      }
+      for (int mb = 0; mb < MBMAX; ++mb)
+        acc[g][mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1[g], x1[mb], acc[g][mb], 0, 0, 0);
   }
   if ((p.K & 63) && kpart == 0) {
     const int k0 = KSF * 64;
     const bool ok = k0 + c4 * 16 < p.K;  // K is a multiple of 16: a chunk is all in or all out
-    v4i w1 = *(const v4i*)(wrow + (ok ? k0 : 0));
-    if (!ok) w1 = (v4i){0, 0, 0, 0};
+    v4i x1[MBMAX];
 #pragma unroll
-    for (int mb = 0; mb < MBMAX; ++mb)
-      acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, *(const v4i*)(xrow[mb] + (ok ? k0 : 0)), acc[mb], 0, 0, 0);
+    for (int mb = 0; mb < MBMAX; ++mb) x1[mb] = *(const v4i*)(xrow[mb] + (ok ? k0 : 0));
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      v4i w1 = *(const v4i*)(wrow[g] + (ok ? k0 : 0));
+      if (!ok) w1 = (v4i){0, 0, 0, 0};
+#pragma unroll
+      for (int mb = 0; mb < MBMAX; ++mb)
+        acc[g][mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, x1[mb], acc[g][mb], 0, 0, 0);
+    }
   }
 
+#ifdef TI_TRACE
+  const uint64_t tr1 = wall_clock64();
+#endif
   if (ksplit > 1) {
 #pragma unroll
-    for (int mb = 0; mb < MBMAX; ++mb)
-      if (mb < MB) *(v4i*)&red[wave][mb][lane * 4] = acc[mb];
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int mb = 0; mb < MBMAX; ++mb)
+        if (mb < MB) *(v4i*)&red[wave][g * MBMAX + mb][lane * 4] = acc[g][mb];
     __syncthreads();
     if (kpart != 0) return;
 #pragma unroll
-    for (int mb = 0; mb < MBMAX; ++mb)
-      if (mb < MB)
-        for (int kp = 1; kp < ksplit; ++kp) acc[mb] += *(const v4i*)&red[wave + kp][mb][lane * 4];
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+      for (int mb = 0; mb < MBMAX; ++mb)
+        if (mb < MB)
+          for (int kp = 1; kp < ksplit; ++kp) acc[g][mb] += *(const v4i*)&red[wave + kp][g * MBMAX + mb][lane * 4];
   }
-  if (slab * 16 >= p.N) return;
 
-  // acc[mb][i]: n = slab*16 + 4*c4 + i, m = mb*16 + r16
-  const EpiCtx e = make_epi(p);
+#ifdef TI_TRACE
+  const uint64_t tr2 = wall_clock64();
+#endif
+  // acc[g][mb][i]: n = (group*G + g)*16 + 4*c4 + i, m = mb*16 + r16
   constexpr int ESZ = OUTCLS == OUT8 ? 1 : (OUTCLS == OUT32 ? 4 : 2);
   char* Cz = (char*)p.C + (int64_t)bz * p.sCb * ESZ;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int n = slab * 16 + 4 * c4 + i;
-    if (n >= p.N) continue;
-    const float col = column_term(e, n);
-    const int bias_i32 = (e.epilogue == TI_EPI_I32 && e.bias_kind == TI_BIAS_I32) ? ((const int*)e.bias)[n] : 0;
+  for (int g = 0; g < G; ++g) {
 #pragma unroll
-    for (int mb = 0; mb < MBMAX; ++mb) {
-      const int m = mb * 16 + r16;
-      if (mb < MB && m < p.M)
-        store_one<OUTCLS>(e, Cz, (int64_t)m * p.sCm + (int64_t)n * p.sCn, acc[mb][i], col, bias_i32, p.out_dtype);
+    for (int i = 0; i < 4; ++i) {
+      const int n = (group * G + g) * 16 + 4 * c4 + i;
+      if (n >= p.N) continue;
+#pragma unroll
+      for (int mb = 0; mb < MBMAX; ++mb) {
+        const int m = mb * 16 + r16;
+        if (mb < MB && m < p.M)
+          store_one<OUTCLS>(e, Cz, (int64_t)m * p.sCm + (int64_t)n * p.sCn, acc[g][mb][i], col[g][i], bias_i32[g][i],
+                            p.out_dtype);
+      }
     }
   }
+#ifdef TI_TRACE
+  if (lane == 0 && blockIdx.x < 1024 && kpart == 0 && (wave / ksplit) == 0) {
+    unsigned long long* tr = ti_trace_buf + blockIdx.x * 8;
+    tr[0] = tr0; tr[1] = tr1; tr[2] = tr2; tr[3] = wall_clock64();
+  }
+#endif
 }
 
 // ---- host side ---------------------------------------------------------------------------------
@@ -1377,6 +1417,7 @@ enum ConfigId {
   CFG_STREAM_256x256,       // persistent: row-major, 16-byte aligned outputs
   CFG_WS_256x128,           // persistent, loads issued by dedicated producer waves
   CFG_STREAM_128x128,
+  CFG_SKINNY_16_G2,  // M <= 16, a wave owns 2 slabs that share its A fragments
 };
 
 static const Config g_configs[] = {
@@ -1391,6 +1432,7 @@ static const Config g_configs[] = {
     TI_STREAM(256, 256, 64, 2, 4, 2, 4, 1),
     TI_WS(256, 128, 128, 2, 2, 1, 3, 4),
     TI_STREAM(128, 128, 64, 2, 2, 2, 3, 2),
+    {"skinny_m16_slab32", {gemm_skinny_kernel<OUT8, 1, 2>, gemm_skinny_kernel<OUT32, 1, 2>, gemm_skinny_kernel<OUT16, 1, 2>}, 16, 32, 64, 512, true, true},
 };
 static const int g_num_configs = (int)(sizeof(g_configs) / sizeof(g_configs[0]));
 
@@ -1531,14 +1573,16 @@ static int run(GemmParams p, int config, hipStream_t stream) {
   if (k.stream_occ && !stream_eligible(p)) return fail(TI_E_COMBO, "config %s needs a row-major output with 16-byte aligned rows", k.name);
   if (k.skinny) {
     if (p.M > k.bm) return fail(TI_E_COMBO, "config %s needs M <= %d", k.name, k.bm);
-    // enough waves to fill the chip: split K between the waves of a workgroup when there are few slabs
-    const int64_t slabs = (int64_t)((p.N + 15) / 16) * p.batch;
+    // a wave owns one group of k.bn rows of B; split K between the waves of a workgroup while
+    // that makes more waves than the chip holds at once and leaves each at least 8 k-steps
+    // (a wave streams slowly: short runs in many waves beat long runs in few)
+    const int64_t groups = (int64_t)((p.N + k.bn - 1) / k.bn) * p.batch;
     const int ksteps = (p.K + 63) / 64;
     int ksplit = 1;
-    while (ksplit < 8 && slabs * ksplit < 4096 && ksplit * 2 <= ksteps) ksplit *= 2;
+    while (ksplit < 8 && groups * ksplit < 4096 && ksteps / (ksplit * 2) >= 8) ksplit *= 2;
     p.ksplit = ksplit;
     const int per_block = 8 / ksplit;
-    dim3 grid((unsigned)(((p.N + 15) / 16 + per_block - 1) / per_block), (unsigned)p.batch, 1);
+    dim3 grid((unsigned)(((p.N + k.bn - 1) / k.bn + per_block - 1) / per_block), (unsigned)p.batch, 1);
     g_last_config = config;
     k.fn[out_class(p.out_dtype)]<<<grid, dim3(k.threads), 0, stream>>>(p);
     return launch_status(k.name);

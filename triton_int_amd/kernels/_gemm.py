@@ -6,31 +6,40 @@ import torch
 from .. import _lib as L
 
 
-def launch_bmm(a3, b3, c3, *, epilogue, bias=None, alpha=None, beta=None, round_mode=L.ROUND_RNE_CLAMP,
-               config=-1):
-    """a3 [B,M,K] int8, b3 [B,N,K] int8 (logical; any strides), c3 [B,M,N] preallocated."""
-    L.require_cuda(a3, b3, c3, bias)
-    assert a3.dtype == torch.int8 and b3.dtype == torch.int8, "operands must be int8"
-    dev = a3.device
-    assert b3.device == dev and c3.device == dev, "operands must be on one device"
-    B, M, K = a3.shape
-    _, N, _ = b3.shape
+def _launch(a, sa, b, sb, c, sc, B, M, N, K, *, epilogue, bias, alpha, beta, round_mode, config):
+    """One ti_bmm_i8_config call: a/b/c are tensors (for pointers, dtype, device), sa/sb/sc the
+    (batch, row, column) element strides of the logical [B,M,K] / [B,N,K] / [B,M,N] views."""
+    L.require_cuda(a, b, c, bias)
+    assert a.dtype == torch.int8 and b.dtype == torch.int8, "operands must be int8"
+    dev = a.device
+    assert b.device == dev and c.device == dev, "operands must be on one device"
     bias_kind = L.BIAS_NONE
+    bias_ptr = 0
     if bias is not None:
         assert bias.device == dev
         assert bias.numel() == N, "bias must have one element per output column"
-        bias = bias.contiguous()
+        if not bias.is_contiguous():
+            bias = bias.contiguous()
         bias_kind = L.TORCH_TO_BIAS[bias.dtype]
-    alpha_t = None if alpha is None else L.scale_tensor(alpha, dev)
-    beta_t = None if beta is None else L.scale_tensor(beta, dev)
-    with torch.cuda.device(dev):
+        bias_ptr = bias.data_ptr()
+    alpha_ptr = 0 if alpha is None else L.scale_tensor(alpha, dev).data_ptr()
+    beta_ptr = 0 if beta is None else L.scale_tensor(beta, dev).data_ptr()
+    with L.on_device(dev):
         rc = L.lib().ti_bmm_i8_config(
-            L.ptr(a3), a3.stride(0), a3.stride(1), a3.stride(2),
-            L.ptr(b3), b3.stride(0), b3.stride(1), b3.stride(2),
-            L.ptr(c3), c3.stride(0), c3.stride(1), c3.stride(2),
-            B, M, N, K, L.ptr(bias), bias_kind, L.ptr(alpha_t), L.ptr(beta_t),
-            int(epilogue), L.TORCH_TO_DT[c3.dtype], int(round_mode), int(config), L.current_stream(dev))
-    L.check(rc, "ti_bmm_i8")
+            a.data_ptr(), sa[0], sa[1], sa[2], b.data_ptr(), sb[0], sb[1], sb[2], c.data_ptr(), sc[0], sc[1], sc[2],
+            B, M, N, K, bias_ptr, bias_kind, alpha_ptr, beta_ptr,
+            int(epilogue), L.TORCH_TO_DT[c.dtype], int(round_mode), int(config), L.current_stream(dev))
+    if rc != 0:
+        L.check(rc, "ti_bmm_i8")
+
+
+def launch_bmm(a3, b3, c3, *, epilogue, bias=None, alpha=None, beta=None, round_mode=L.ROUND_RNE_CLAMP,
+               config=-1):
+    """a3 [B,M,K] int8, b3 [B,N,K] int8 (logical; any strides), c3 [B,M,N] preallocated."""
+    B, M, K = a3.shape
+    _, N, _ = b3.shape
+    _launch(a3, a3.stride(), b3, b3.stride(), c3, c3.stride(), B, M, N, K, epilogue=epilogue, bias=bias,
+            alpha=alpha, beta=beta, round_mode=round_mode, config=config)
     return c3
 
 
@@ -50,8 +59,8 @@ def linear(a, w, *, epilogue, out_dtype, bias=None, alpha=None, beta=None, out=N
     else:
         assert out.dtype == out_dtype and out.numel() == M * N, "out has the wrong dtype or size"
         c = out.view(M, N)
-    launch_bmm(a.unsqueeze(0), w.unsqueeze(0), c.unsqueeze(0), epilogue=epilogue, bias=bias, alpha=alpha,
-               beta=beta, round_mode=round_mode, config=config)
+    _launch(a, (0, a.stride(0), a.stride(1)), w, (0, w.stride(0), w.stride(1)), c, (0, c.stride(0), c.stride(1)),
+            1, M, N, K, epilogue=epilogue, bias=bias, alpha=alpha, beta=beta, round_mode=round_mode, config=config)
     return c.view(*tmp_shape, N)
 
 

@@ -44,7 +44,7 @@ def layer_norm_fwd_fused_single_pass_q(x, weight, bias, eps, use_rms_norm=False,
     if _return_stats:
         mean = torch.empty(M, dtype=torch.float32, device=x.device)
         rstd = torch.empty(M, dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
+    with L.on_device(x.device):
         rc = L.lib().ti_layernorm_q(L.ptr(a_arg), a_arg.stride(0) if M > 1 else N, L.ptr(weight), L.ptr(bias),
                                     float(eps), L.ptr(o2), N, M, N, int(bool(use_rms_norm)), int(_round_mode),
                                     L.ptr(mean), L.ptr(rstd), L.current_stream(x.device))
@@ -83,7 +83,7 @@ def dq_add_layernorm_q(input_int32, input_scale_fp, residual_input_fp, gamma, be
         rstd = torch.empty(rows, dtype=torch.float32, device=dev)
     if torch.is_tensor(input_scale_fp):
         input_scale_fp = float(input_scale_fp)  # the module holds a python float (nn/fused.py:62)
-    with torch.cuda.device(dev):
+    with L.on_device(dev):
         rc = L.lib().ti_dq_add_layernorm_q(
             L.ptr(acc), acc.stride(0) if rows > 1 else H, float(input_scale_fp), L.ptr(rin),
             rin.stride(0) if rows > 1 else H, L.ptr(gamma), L.ptr(beta), float(eps), L.ptr(rout), H, L.ptr(y), H,
@@ -99,7 +99,7 @@ def gelu_q(x, scale, *, _round_mode=L.ROUND_RNE_CLAMP):
     x = x.to(torch.float32).contiguous()
     y = torch.empty(x.shape, dtype=torch.int8, device=x.device)
     s = L.scale_tensor(scale, x.device)
-    with torch.cuda.device(x.device):
+    with L.on_device(x.device):
         rc = L.lib().ti_gelu_q(L.ptr(x), L.ptr(s), L.ptr(y), x.numel(), int(_round_mode), L.current_stream(x.device))
     L.check(rc, "ti_gelu_q")
     return y
@@ -119,7 +119,7 @@ def softmax_q(x, scale, causal_q_len=0):
     rows = x2.shape[0]
     y = torch.empty(x.shape, dtype=torch.int8, device=x.device)
     y2 = y.view(-1, cols)
-    with torch.cuda.device(x.device):
+    with L.on_device(x.device):
         rc = L.lib().ti_softmax_q(L.ptr(x2), x2.stride(0) if rows > 1 else cols, float(scale), L.ptr(y2), cols, rows,
                                   cols, int(causal_q_len), L.current_stream(x.device))
     L.check(rc, "ti_softmax_q")
