@@ -1480,6 +1480,10 @@ static bool stream_eligible(const GemmParams& p) {
 // go to them; the rest to the one-tile kernels.
 static int pick_config(const GemmParams& p) {
   if (!fast_eligible(p)) return CFG_GATHER;
+  if (p.M <= 16) {
+    // two slabs per wave halve the A re-reads; worth it only while enough waves remain (measured)
+    return (p.N + 31) / 32 >= 160 ? CFG_SKINNY_16_G2 : CFG_SKINNY_16;
+  }
   if (p.M <= 64) return CFG_SKINNY_16 + (p.M > 16) + (p.M > 32);
   const bool stream = stream_eligible(p);
   // short K: the epilogue dominates and the larger tile halves the operand traffic per output
