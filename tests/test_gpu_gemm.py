@@ -339,6 +339,29 @@ def test_decode_shapes_skinny_kernel(M, N, K):
     assert mx <= 1 and rate < 1e-3
 
 
+@pytest.mark.parametrize("M,N,K", [(16, 5136, 1104), (9, 400, 2048), (1, 48, 64), (13, 5120, 5120)])
+def test_every_skinny_config_ragged_shapes(M, N, K):
+    """Each weight-streaming configuration (one or two 16-row slabs per wave) forced on shapes whose
+    N is not a multiple of the slab group, whose K has left-over k-steps and a 16-byte tail."""
+    linear, _, _ = _kl()
+    g = rng(M + N + K)
+    a, w = rand_i8(g, M, K, lo=-128), rand_i8(g, N, K, lo=-128)
+    b32 = g.integers(-2**20, 2**20, size=N, dtype=np.int32)
+    b8 = rand_i8(g, N)
+    ga, gw = gpu(a), gpu(w)
+    want32 = O.linear_a8_w8_b32_o32(a, w, b32)
+    alpha = np.float32(40.0 / (np.sqrt(K) * 127 * 127 / 3)); beta = np.float32(0.05)
+    want8 = O.linear_a8_w8_b8_o8(a, w, b8, alpha, beta)
+    ran = 0
+    for cfg, name in _configs(M):
+        if not name.startswith("skinny"):
+            continue
+        ran += 1
+        assert np.array_equal(cpu(linear.linear_a8_w8_b32_o32(ga, gw, gpu(b32), _config=cfg)), want32), name
+        assert np.array_equal(cpu(linear.linear_a8_w8_b8_o8(ga, gw, gpu(b8), alpha, beta, _config=cfg)), want8), name
+    assert ran >= 4
+
+
 def test_decode_attention_bmms():
     """16 query tokens against a 2048-long int8 KV, 40 heads of 128 (OPT-13B decode)."""
     _, bmm, _ = _kl()
