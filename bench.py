@@ -224,6 +224,27 @@ def extras(torch, dev):
     del p
     for v in out.values():
         v["frac_hbm_peak"] = v["GBps"] / HBM_PEAK_GBPS
+    # config 1: one W8A8B8O8Linear 512 x 768 x 768 (launch-latency sized: no roofline claim).  Eager
+    # time includes the Python launch path; the graph replay is the kernel alone.
+    from triton_int_amd.kernels import linear
+
+    x1 = torch.randint(-127, 128, (512, 768), dtype=torch.int8, device=dev)
+    w1 = torch.randint(-127, 128, (768, 768), dtype=torch.int8, device=dev)
+    b1 = torch.randint(-127, 128, (768,), dtype=torch.int8, device=dev)
+    al, be = torch.tensor(0.0021, device=dev), torch.tensor(0.013, device=dev)
+    o1 = torch.empty((512, 768), dtype=torch.int8, device=dev)
+    eager_ms = time_region(torch, lambda: linear.linear_a8_w8_b8_o8(x1, w1, b1, al, be, out=o1), 200, 20)
+    graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        linear.linear_a8_w8_b8_o8(x1, w1, b1, al, be, out=o1)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(20):
+                linear.linear_a8_w8_b8_o8(x1, w1, b1, al, be, out=o1)
+    torch.cuda.synchronize()
+    graph_ms = time_region(torch, graph.replay, 20, 3) / 20
+    out["single_linear_512x768x768"] = {"eager_us": eager_ms * 1e3, "graph_us": graph_ms * 1e3,
+                                        "TOPS_graph": 2.0 * 512 * 768 * 768 / (graph_ms * 1e-3) / 1e12}
     return out
 
 
@@ -242,6 +263,34 @@ def decoder_layer_ms(torch, dev):
         layers[state["i"]](x)
 
     out = {"prefill_1x2048_ms": time_region(torch, prefill, 10, 2)}
+    # per-op breakdown of the prefill: each stage on the tensors a traced forward produced, timed alone
+    from triton_int_amd.kernels.bmm import bmm_s8t_s8n_s8t
+    from triton_int_amd.kernels.fused import softmax_q
+
+    tr, L0 = {}, layers[0]
+    L0(x, _trace=tr)
+    ctx_v = torch.empty_like(tr["ctx"])
+    stages = {
+        "ln1_layernorm_q": lambda: L0.ln1(x),
+        "qkv_3x_linear_o8": lambda: (L0.q_proj(tr["h8"]), L0.k_proj(tr["h8"]), L0.v_proj(tr["h8"])),
+        "qk_bmm_o8": lambda: bmm_s8t_s8n_s8t(tr["q"], tr["k_all"], L0.qk_alpha, out=tr["scores"]),
+        "softmax_q_causal": lambda: softmax_q(tr["scores"], L0.score_scale, causal_q_len=2048),
+        "pv_bmm_o8": lambda: bmm_s8t_s8n_s8t(tr["probs"], tr["vt_all"], L0.pv_alpha,
+                                             out=ctx_v[0].view(2048, 40, 128).transpose(0, 1)),
+        "out_proj_linear_o32": lambda: L0.out_proj(tr["ctx"]),
+        "ln2_dq_add_layernorm_q": lambda: L0.ln2(x, tr["acc"]),
+        "fc1_linear_gelu_q": lambda: L0.fc1(tr["h8b"]),
+        "fc2_linear_f32": lambda: L0.fc2(tr["f8"]),
+    }
+    br = {k: time_region(torch, f, 10, 2) for k, f in stages.items()}
+    br["glue_head_split_transpose_residual_add"] = max(0.0, out["prefill_1x2048_ms"] - sum(br.values()))
+    out["prefill_breakdown_ms"] = br
+    # ideal: GEMM/BMM ops at the 5.0 POP/s peak, row kernels at 8 TB/s on their algorithmic bytes
+    S_, H_, F_ = 2048, 5120, 20480
+    ideal = 1374.4e9 / 5.0e15 + (S_ * H_ * 5 + S_ * H_ * 13 + 40 * S_ * S_ * 2) / 8.0e12
+    out["prefill_ideal_ms"] = ideal * 1e3
+    out["prefill_ideal_over_measured"] = ideal * 1e3 / out["prefill_1x2048_ms"]
+    del tr, ctx_v
     kc = torch.randint(-127, 128, (40, 2048, 128), dtype=torch.int8, device=dev)
     vc = torch.randint(-127, 128, (40, 128, 2048), dtype=torch.int8, device=dev)
     xd = torch.randn((1, 16, 5120), device=dev)
@@ -333,6 +382,8 @@ def main():
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
     dom_ms = sum(a.elapsed_time(b) for a, b in events) / args.steps  # per step, all launches of the dominant kernel
+    # device time of whole steps: start event of step i to start event of step i+1
+    step_ms = sorted(events[i][0].elapsed_time(events[i + 1][0]) for i in range(args.steps - 1))
     dom_ops = sum(o for *_, o in groups[dominant])
     achieved = dom_ops / (dom_ms * 1e-3) / 1e12
 
@@ -344,6 +395,8 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": ms_per_step,
+        "ms_per_step_device_p20_p50_p80": ([step_ms[int(q * (len(step_ms) - 1))] for q in (0.2, 0.5, 0.8)]
+                                           if step_ms else None),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

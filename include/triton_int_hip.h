@@ -192,6 +192,17 @@ int ti_gelu_q(const float* x, const float* scale, int8_t* y, int64_t n,
 int ti_softmax_q(const int8_t* x, int64_t x_row_stride, float scale,
                  int8_t* y, int64_t y_row_stride, int rows, int cols, int causal_q_len, void* stream);
 
+/*
+ * dst[c, r] = src[r, c] for an int8 matrix of `rows` x `cols` (row strides in elements, unit column
+ * stride on both sides).  The P.V BMM wants V^T with the sequence as its contiguous dimension
+ * (bmm_s8t_s8n_*, kernels/bmm.py:428-464 takes b as [B, N, K]); callers of the reference's modules
+ * build it with `v.transpose(1, 2).contiguous()` in torch.  With src = V [S, heads*D] and
+ * dst = V^T viewed as [heads*D, T] (dst pointing at column T - S) this writes every head's V^T, or
+ * appends S positions to a KV cache, in one launch.
+ */
+int ti_transpose_i8(const int8_t* src, int64_t src_row_stride, int8_t* dst, int64_t dst_row_stride,
+                    int rows, int cols, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

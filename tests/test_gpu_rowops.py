@@ -168,3 +168,25 @@ def test_softmax_q(rows, cols, q_len):
         assert got.min() >= 0
     x3 = x.reshape(1, rows, cols)
     assert fused.softmax_q(gpu(x3), 0.05).shape == (1, rows, cols)
+
+
+@pytest.mark.parametrize("rows,cols", [(2048, 5120), (16, 5120), (1, 128), (70, 33), (64, 64), (129, 257)])
+def test_transpose_i8(rows, cols):
+    """Pure data movement: the checker is numpy's transpose.  Covers whole tiles, ragged edges,
+    unaligned sizes, and the KV-cache form (writing the last `rows` columns of a wider matrix)."""
+    fused = _fused()
+    g = rng(rows * 3 + cols)
+    x = g.integers(-128, 128, size=(rows, cols), dtype=np.int8)
+    got = cpu(fused.transpose_i8(gpu(x)))
+    assert got.shape == (cols, rows) and np.array_equal(got, x.T)
+    # source with a row pitch (a column slice of a wider matrix)
+    wide = g.integers(-128, 128, size=(rows, cols + 48), dtype=np.int8)
+    got = cpu(fused.transpose_i8(gpu(wide)[:, 16:16 + cols]))
+    assert np.array_equal(got, wide[:, 16:16 + cols].T)
+    # destination = the last `rows` columns of a [cols, T] cache; the rest must stay untouched
+    T = rows + 37
+    cache = g.integers(-128, 128, size=(cols, T), dtype=np.int8)
+    gc = gpu(cache)
+    fused.transpose_i8(gpu(x), out=gc[:, T - rows:])
+    want = cache.copy(); want[:, T - rows:] = x.T
+    assert np.array_equal(cpu(gc), want)

@@ -398,6 +398,50 @@ __global__ __launch_bounds__(GQ_THREADS) void gelu_q_any_kernel(const float* x, 
     y[i] = (int8_t)q8(gelu_tanh_scaled(x[i], s), round_mode);
 }
 
+// ---- int8 2-D transpose ------------------------------------------------------------------------
+// dst[c, r] = src[r, c].  64 x 64-byte tiles through LDS: 16-byte loads along the source rows,
+// 16-byte stores along the destination rows (4 lanes cover a 64-byte run on both sides).
+constexpr int TR_TILE = 64, TR_PITCH = TR_TILE + 4;
+
+__global__ __launch_bounds__(256) void transpose_i8_kernel(const int8_t* __restrict__ src, int64_t src_rs,
+                                                           int8_t* __restrict__ dst, int64_t dst_rs, int rows, int cols,
+                                                           int vec_src, int vec_dst) {
+  __shared__ __attribute__((aligned(16))) int8_t tile[TR_TILE][TR_PITCH];
+  const int t = threadIdx.x;
+  const int r0 = blockIdx.y * TR_TILE, c0 = blockIdx.x * TR_TILE;
+  {
+    const int r = t >> 2, cc = (t & 3) * 16;  // source row, first column of this thread's 16 bytes
+    unsigned w[4] = {0u, 0u, 0u, 0u};
+    if (r0 + r < rows) {
+      const int8_t* sp = src + (int64_t)(r0 + r) * src_rs + c0 + cc;
+      if (vec_src && c0 + cc + 16 <= cols) {
+        const v4u v = *(const v4u*)sp;
+        w[0] = v[0]; w[1] = v[1]; w[2] = v[2]; w[3] = v[3];
+      } else {
+        for (int i = 0; i < 16; ++i)
+          if (c0 + cc + i < cols) w[i >> 2] |= (unsigned)(uint8_t)sp[i] << ((i & 3) * 8);
+      }
+    }
+#pragma unroll
+    for (int g = 0; g < 4; ++g) *(unsigned*)&tile[r][cc + 4 * g] = w[g];
+  }
+  __syncthreads();
+  {
+    const int c = t >> 2, rr = (t & 3) * 16;  // destination row (source column), first of 16 source rows
+    if (c0 + c >= cols) return;
+    unsigned w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 16; ++i) w[i >> 2] |= (unsigned)(uint8_t)tile[rr + i][c] << ((i & 3) * 8);
+    int8_t* dp = dst + (int64_t)(c0 + c) * dst_rs + r0 + rr;
+    if (vec_dst && r0 + rr + 16 <= rows) {
+      *(v4u*)dp = (v4u){w[0], w[1], w[2], w[3]};
+    } else {
+      for (int i = 0; i < 16; ++i)
+        if (r0 + rr + i < rows) dp[i] = (int8_t)(w[i >> 2] >> ((i & 3) * 8));
+    }
+  }
+}
+
 }  // namespace ti
 
 extern "C" {
@@ -485,6 +529,22 @@ int ti_gelu_q(const float* x, const float* scale, int8_t* y, int64_t n, int roun
     rc = ti::launch_status("gelu_q_any_kernel");
   }
   return rc;
+}
+
+int ti_transpose_i8(const int8_t* src, int64_t src_row_stride, int8_t* dst, int64_t dst_row_stride, int rows,
+                    int cols, void* stream) {
+  if (rows < 0 || cols < 0) return ti::fail(TI_E_SHAPE, "negative size");
+  if (rows == 0 || cols == 0) return TI_OK;
+  if (!src || !dst) return ti::fail(TI_E_NULL, "src and dst are required");
+  int rc = ti::check_device();
+  if (rc != TI_OK) return rc;
+  const int vec_src = ((((uintptr_t)src) | (uintptr_t)(src_row_stride)) & 15) == 0;
+  const int vec_dst = ((((uintptr_t)dst) | (uintptr_t)(dst_row_stride)) & 15) == 0;
+  dim3 grid((unsigned)((cols + ti::TR_TILE - 1) / ti::TR_TILE), (unsigned)((rows + ti::TR_TILE - 1) / ti::TR_TILE));
+  if (grid.y > 65535) return ti::fail(TI_E_SHAPE, "more than 65535 * 64 rows");
+  ti::transpose_i8_kernel<<<grid, dim3(256), 0, (hipStream_t)stream>>>(src, src_row_stride, dst, dst_row_stride, rows,
+                                                                    cols, vec_src, vec_dst);
+  return ti::launch_status("transpose_i8_kernel");
 }
 
 }  // extern "C"

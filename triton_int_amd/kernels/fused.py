@@ -124,3 +124,20 @@ def softmax_q(x, scale, causal_q_len=0):
                                   cols, int(causal_q_len), L.current_stream(x.device))
     L.check(rc, "ti_softmax_q")
     return y
+
+
+def transpose_i8(src, out=None):
+    """int8 [rows, cols] (unit column stride) -> [cols, rows].  `out` may be any int8 view of that
+    shape with unit column stride, e.g. the last `rows` columns of a V^T cache [heads*D, T].  The
+    reference's callers do this step with torch (`transpose(...).contiguous()`)."""
+    L.require_cuda(src, out)
+    assert src.dtype == torch.int8 and src.dim() == 2 and src.stride(1) == 1, "src must be int8 [rows, cols], unit column stride"
+    rows, cols = src.shape
+    if out is None:
+        out = torch.empty((cols, rows), dtype=torch.int8, device=src.device)
+    assert out.dtype == torch.int8 and tuple(out.shape) == (cols, rows) and (out.stride(1) == 1 or rows == 1)
+    with L.on_device(src.device):
+        rc = L.lib().ti_transpose_i8(L.ptr(src), src.stride(0), L.ptr(out), out.stride(0), rows, cols,
+                                     L.current_stream(src.device))
+    L.check(rc, "ti_transpose_i8")
+    return out

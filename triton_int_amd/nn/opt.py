@@ -21,7 +21,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels.bmm import bmm_s8t_s8n_s8t
-from ..kernels.fused import softmax_q
+from ..kernels.fused import softmax_q, transpose_i8
 from .fused import DQ_Add_LayerNorm_Q, LayerNormQ, W8A8BFP32OFP32_GeLu_Q
 from .linear import W8A8B8O8Linear, W8A8B32O32LinearWithoutScaling, W8A8BFP32OFP32Linear
 
@@ -72,7 +72,10 @@ class W8A8OPTDecoderLayer(torch.nn.Module):
         return self
 
     def _heads(self, t, B, S):
-        # [B,S,H] int8 -> [B*heads, S, D] (a copy: the BMM wants each head's rows contiguous in K)
+        # [B,S,H] int8 -> [B*heads, S, D].  One batch: a strided view (the BMM takes row and batch
+        # strides, each head's rows stay K-contiguous).  Several batches: a copy.
+        if B == 1:
+            return t.view(S, self.heads, self.head_dim).transpose(0, 1)
         return t.view(B, S, self.heads, self.head_dim).transpose(1, 2).reshape(B * self.heads, S, self.head_dim)
 
     @torch.no_grad()
@@ -85,14 +88,18 @@ class W8A8OPTDecoderLayer(torch.nn.Module):
         h8 = self.ln1(hidden)
         q = self._heads(self.q_proj(h8), B, S)
         k_new = self._heads(self.k_proj(h8), B, S)
-        v_new = self._heads(self.v_proj(h8), B, S)
+        v = self.v_proj(h8)                                                        # [B,S,H] int8
         if kv_cache is None:
-            k_all, vt_all = k_new, v_new.transpose(1, 2).contiguous()
+            k_all = k_new
+            vt_all = torch.empty((B * self.heads, self.head_dim, S), dtype=torch.int8, device=hidden.device)
         else:
             k_all, vt_all = kv_cache
             T = k_all.shape[1]
             k_all[:, T - S:, :] = k_new
-            vt_all[:, :, T - S:] = v_new.transpose(1, 2)
+        T = vt_all.shape[2]
+        # V^T of every head of a batch in one transpose: [S, heads*D] -> the last S columns of [heads*D, T]
+        for b in range(B):
+            transpose_i8(v[b], out=vt_all[b * self.heads:(b + 1) * self.heads].view(H, T)[:, T - S:])
         T = k_all.shape[1]
         scores = bmm_s8t_s8n_s8t(q, k_all, self.qk_alpha)                           # [B*heads, S, T] int8
         probs = softmax_q(scores, self.score_scale, causal_q_len=S if self.causal else 0)
