@@ -54,12 +54,12 @@ def test_gpu_gemm_fixture_all_epilogues_and_configs():
     al, be = float(d["alpha"]), float(d["beta"])
     for cfg in range(-1, _lib.lib().ti_gemm_num_configs()):
         name = _lib.lib().ti_gemm_config_name(cfg).decode() if cfg >= 0 else ""
-        if name.startswith("skinny") and int(name.split("_")[1][1:]) < d["a"].shape[0]:
+        if name.startswith(("skinny", "rows4")) and int(name.split("_")[1][1:]) < d["a"].shape[0]:
             continue  # that configuration takes fewer activation rows than the fixture has
         assert np.array_equal(_host(linear.linear_a8_w8_b32_o32(a, w, _dev(d["b32"]), _config=cfg)), d["o32"])
         assert np.array_equal(_host(linear.linear_a8_w8_b32_o32_with_scaling(a, w, _dev(d["b32"]), 0.01, be, _config=cfg)), d["o32_scaled"])
         for name, rm in (("rne", 0), ("trunc", 1)):
-            if rm == 1 and cfg > 0 and not name.startswith("skinny"):
+            if rm == 1 and cfg > 0 and not name.startswith(("skinny", "rows4")):
                 continue  # truncation (test-time switch) is not implemented by the large-tile kernels
             assert np.array_equal(_host(linear.linear_a8_w8_b8_o8(a, w, _dev(d["b8"]), al, be, _round_mode=rm, _config=cfg)), d[f"o8_{name}"])
             assert np.array_equal(_host(linear.linear_relu_a8_w8_b8_o8(a, w, _dev(d["b8"]), al, be, _round_mode=rm, _config=cfg)), d[f"o8_relu_{name}"])

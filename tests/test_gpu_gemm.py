@@ -24,7 +24,7 @@ def _configs(M=1, N=None, out8=False):
     n = L.lib().ti_gemm_num_configs()
     out = [(i, L.lib().ti_gemm_config_name(i).decode()) for i in range(n)]
     def fits(nm):  # "skinny_m<rows>_..." configurations take at most <rows> activation rows
-        if nm.startswith("skinny"):
+        if nm.startswith(("skinny", "rows4")):
             return M <= int(nm.split("_")[1][1:])
         if nm.startswith(("stream", "ws_")) and out8:
             return N is not None and N % 16 == 0
@@ -325,7 +325,7 @@ def test_decode_shapes_skinny_kernel(M, N, K):
     b8 = rand_i8(g, N); bf = g.standard_normal(N).astype(np.float32)
     ga, gw = gpu(a), gpu(w)
     got = cpu(linear.linear_a8_w8_b32_o32(ga, gw, gpu(b32)))
-    assert L.lib().ti_gemm_config_name(L.lib().ti_gemm_last_config()).decode().startswith("skinny")
+    assert L.lib().ti_gemm_config_name(L.lib().ti_gemm_last_config()).decode().startswith(("skinny", "rows4"))
     assert np.array_equal(got, O.linear_a8_w8_b32_o32(a, w, b32))
     alpha = np.float32(40.0 / (np.sqrt(K) * 127 * 127 / 3)); beta = np.float32(0.05)
     assert np.array_equal(cpu(linear.linear_a8_w8_b8_o8(ga, gw, gpu(b8), alpha, beta)), O.linear_a8_w8_b8_o8(a, w, b8, alpha, beta))
@@ -354,7 +354,7 @@ def test_every_skinny_config_ragged_shapes(M, N, K):
     want8 = O.linear_a8_w8_b8_o8(a, w, b8, alpha, beta)
     ran = 0
     for cfg, name in _configs(M):
-        if not name.startswith("skinny"):
+        if not name.startswith(("skinny", "rows4")):
             continue
         ran += 1
         assert np.array_equal(cpu(linear.linear_a8_w8_b32_o32(ga, gw, gpu(b32), _config=cfg)), want32), name

@@ -1365,6 +1365,167 @@ __global__ __launch_bounds__(512, UU ? 2 : 4) void gemm_skinny_kernel(GemmParams
 #endif
 }
 
+// ---- decode kernel: M <= 16, weights streamed as whole 1 KB row pieces ----------------------------
+//
+// With 16 or fewer activation rows the GEMM is a read of the weight matrix, and what decides its
+// speed is how the reads reach HBM.  Loading MFMA operands directly (16 rows x 64 bytes per
+// instruction, gemm_skinny_kernel) scatters every wave's requests over 16 rows one row pitch
+// apart.  Here a wave owns groups of 4 consecutive weight rows and copies them global -> LDS in
+// 1 KB row pieces (one instruction = 64 lanes x 16 consecutive bytes), 3 stages of 4 x 1 KB in
+// flight per wave, and the waves of the chip together sweep the matrix almost linearly.  The
+// activations (16 x K bytes) are staged in LDS once per workgroup by a ninth wave, 1 KB of K at
+// a time, three chunks deep, and shared by the 8 consumer waves; a barrier per chunk hands them
+// over.  Operand fragments then come from LDS: rows 4..15 of the 16-row MFMA operand repeat rows
+// 0..3 (their results are dropped), so no K split and no reduction between waves is needed.
+constexpr int R4_NW = 8, R4_RG = 4, R4_KC = 1024, R4_PITCH = R4_KC + 16, R4_NST = 3, R4_XB = 3, R4_UMAX = 4;
+
+template <int OUTCLS>
+__global__ __launch_bounds__((R4_NW + 1) * 64) void gemm_rows4_kernel(GemmParams p) {
+  constexpr int STAGE = R4_RG * R4_PITCH;  // one job: 4 rows x 1 KB (+ padding against bank conflicts)
+  constexpr int XBUF = 16 * R4_PITCH;
+  __shared__ __attribute__((aligned(16))) char lds[R4_XB * XBUF + R4_NW * R4_NST * STAGE];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int bz = blockIdx.y;
+  const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+  const int OOB = (int)0x80000000;
+  const int lda = (int)p.sAm, ldb = (int)p.sBn;
+  const int NCH = (p.K + R4_KC - 1) / R4_KC;  // chunks of K
+  // KS = 2 (few weight rows): two waves share a unit and take the even / the odd chunks of K, so
+  // that all 8 waves stream; their partial sums meet in LDS at the end.  Only with a single pass.
+  const int KS = p.ksplit;
+  const int NSLOT = R4_NW / KS;  // units a workgroup works on at a time
+  // units (groups of 4 weight rows) of this workgroup: [ub0, ub1), dealt to the slots round-robin,
+  // at most NSLOT * R4_UMAX of them per pass over K
+  const int NU = (p.N + R4_RG - 1) / R4_RG;
+  const int per = (NU + (int)gridDim.x - 1) / (int)gridDim.x;
+  const int ub0 = min(NU, (int)blockIdx.x * per), ub1 = min(NU, ub0 + per);
+  const int npass = max(1, (ub1 - ub0 + NSLOT * R4_UMAX - 1) / (NSLOT * R4_UMAX));
+  const int kl = lane * 16;  // this lane's byte inside a 1 KB piece
+
+  if (wave == R4_NW) {
+    // ---- activation producer: chunk g (counted over all passes) goes to buffer g % 3
+    const v4i rX = make_rsrc(p.A + (int64_t)bz * p.sAb, (p.M - 1) * lda + p.K);
+    const int total = npass * NCH;
+    auto issue_x = [&](int g) {
+      const int k0 = (g % NCH) * R4_KC;
+      const bool in = g < total && k0 + kl < p.K;
+      const unsigned dst = lds_base + (g % R4_XB) * XBUF;
+#pragma unroll
+      for (int m = 0; m < 16; ++m)
+        dma16_to_lds(rX, in ? min(m, p.M - 1) * lda + kl : OOB, k0, dst + m * R4_PITCH);
+    };
+    issue_x(0);
+    issue_x(1);
+    for (int g = 0; g < total; ++g) {
+      wait_loads_and_barrier<16>();  // chunk g has landed (chunk g+1 may be in flight); hand it over
+      issue_x(g + 2);                // into the buffer of chunk g-1, whose readers passed the barrier
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (KS > 1) asm volatile("s_barrier" ::: "memory");  // the consumers' reduction barrier
+    return;
+  }
+
+  // ---- consumers
+  const int slot = wave % NSLOT, kpart = wave / NSLOT;
+  const v4i rW = make_rsrc(p.B + (int64_t)bz * p.sBb, (p.N - 1) * ldb + p.K);
+  const unsigned ring = lds_base + R4_XB * XBUF + wave * (R4_NST * STAGE);
+  char* ring_p = lds + R4_XB * XBUF + wave * (R4_NST * STAGE);
+  const int r16 = lane & 15, c4 = lane >> 4;
+  const int w_lane = (r16 & (R4_RG - 1)) * R4_PITCH + c4 * 16;  // rows 4..15 of the operand repeat rows 0..3
+  const int x_lane = r16 * R4_PITCH + c4 * 16;
+  const EpiCtx e = make_epi(p);
+  constexpr int ESZ = OUTCLS == OUT8 ? 1 : (OUTCLS == OUT32 ? 4 : 2);
+  char* Cz = (char*)p.C + (int64_t)bz * p.sCb * ESZ;
+  const int nch_mine = (NCH - kpart + KS - 1) / KS;  // chunks kpart, kpart + KS, ...
+
+  int g = 0;  // chunk counter over all passes (selects the activation buffer)
+  for (int pass = 0; pass < npass; ++pass) {
+    const int u_first = ub0 + pass * (NSLOT * R4_UMAX) + slot;  // this wave's units: u_first + NSLOT*i, i < nu
+    const int u_end = min(ub1, ub0 + (pass + 1) * (NSLOT * R4_UMAX));
+    const int nu = u_first < u_end ? (u_end - u_first + NSLOT - 1) / NSLOT : 0;
+    const int njobs = nu * nch_mine;
+    // job j = (this wave's chunk number j / nu, unit j % nu): 4 loads of 1 KB, into ring slot j % 3;
+    // beyond the last job the loads are redirected out of range (zeros into a slot nobody reads)
+    // so that the number in flight stays constant
+    auto issue_job = [&](int j) {
+      const bool real = j < njobs;
+      const int cm = real ? j / nu : 0, ui = real ? j - cm * nu : 0;
+      const int k0 = (kpart + cm * KS) * R4_KC;
+      const int row0 = (u_first + ui * NSLOT) * R4_RG;
+      const bool in = real && k0 + kl < p.K;
+      const unsigned dst = ring + (j % R4_NST) * STAGE;
+#pragma unroll
+      for (int r = 0; r < R4_RG; ++r)
+        dma16_to_lds(rW, in ? min(row0 + r, p.N - 1) * ldb + kl : OOB, k0, dst + r * R4_PITCH);
+    };
+    v4i acc[R4_UMAX];
+#pragma unroll
+    for (int i = 0; i < R4_UMAX; ++i) acc[i] = (v4i){0, 0, 0, 0};
+    if (nu > 0) {
+      issue_job(0);
+      issue_job(1);
+    }
+    int j = 0;
+    for (int c = 0; c < NCH; ++c, ++g) {
+      asm volatile("s_barrier" ::: "memory");  // activation chunk g is in LDS
+      if (nu == 0 || c % KS != kpart) continue;
+      // the chunk's 16 activation fragments are read once and serve all of the wave's units
+      // (bytes past K were loaded as zeros, so all 16 k-steps can always be used)
+      const char* xb = lds + (g % R4_XB) * XBUF + x_lane;
+      v4i xf[16];
+#pragma unroll
+      for (int s = 0; s < 16; ++s) xf[s] = *(const v4i*)(xb + s * 64);
+#pragma unroll
+      for (int ui = 0; ui < R4_UMAX; ++ui) {
+        if (ui < nu) {
+          issue_job(j + 2);
+          asm volatile("s_waitcnt vmcnt(%0)" ::"n"(R4_RG * (R4_NST - 1)) : "memory");  // job j has landed
+          const char* wb = ring_p + (j % R4_NST) * STAGE + w_lane;
+#pragma unroll
+          for (int s = 0; s < 16; ++s)
+            acc[ui] = __builtin_amdgcn_mfma_i32_16x16x64_i8(*(const v4i*)(wb + s * 64), xf[s], acc[ui], 0, 0, 0);
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // slot j % 3 is free for job j + 3
+          ++j;
+        }
+      }
+    }
+    if (nu > 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // trailing redirected loads
+    if (KS > 1) {
+      // odd-chunk waves park their sums in their own (now idle) ring; the even-chunk partner adds them
+      if (kpart == 1) {
+#pragma unroll
+        for (int ui = 0; ui < R4_UMAX; ++ui)
+          if (ui < nu) *(v4i*)(ring_p + ui * 1024 + lane * 16) = acc[ui];
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      if (kpart == 1) return;
+      const char* other = ring_p + NSLOT * (R4_NST * STAGE);
+#pragma unroll
+      for (int ui = 0; ui < R4_UMAX; ++ui)
+        if (ui < nu) acc[ui] += *(const v4i*)(other + ui * 1024 + lane * 16);
+    }
+    // acc[ui][i], lanes 0..15: n = unit*4 + i, m = lane
+    if (c4 == 0 && r16 < p.M) {
+#pragma unroll
+      for (int ui = 0; ui < R4_UMAX; ++ui) {
+        if (ui < nu) {
+          const int n0 = (u_first + ui * NSLOT) * R4_RG;
+#pragma unroll
+          for (int i = 0; i < R4_RG; ++i) {
+            const int n = n0 + i;
+            if (n < p.N) {
+              const int bias_i32 = (e.epilogue == TI_EPI_I32 && e.bias_kind == TI_BIAS_I32) ? ((const int*)e.bias)[n] : 0;
+              store_one<OUTCLS>(e, Cz, (int64_t)r16 * p.sCm + (int64_t)n * p.sCn, acc[ui][i], column_term(e, n), bias_i32,
+                                p.out_dtype);
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
 // ---- host side ---------------------------------------------------------------------------------
 
 typedef void (*KernelFn)(GemmParams);
@@ -1376,6 +1537,7 @@ struct Config {
   bool fast;       // needs the aligned K-contiguous layout
   bool skinny = false;  // gemm_skinny_kernel: M <= 64, grid over 16-row slabs of B
   int stream_occ = 0;   // > 0: gemm_mfma_stream_kernel, this many workgroups per CU walk the tile list
+  bool rows4 = false;   // gemm_rows4_kernel: M <= 16
 };
 
 #define TI_FAST(BM, BN, BK, WM, WN, SWZ, NS)                                              \
@@ -1418,6 +1580,7 @@ enum ConfigId {
   CFG_WS_256x128,           // persistent, loads issued by dedicated producer waves
   CFG_STREAM_128x128,
   CFG_SKINNY_16_G2,  // M <= 16, a wave owns 2 slabs that share its A fragments
+  CFG_ROWS4_16,      // M <= 16, K >= 1024: weights streamed as 1 KB row pieces
 };
 
 static const Config g_configs[] = {
@@ -1433,6 +1596,7 @@ static const Config g_configs[] = {
     TI_WS(256, 128, 128, 2, 2, 1, 3, 4),
     TI_STREAM(128, 128, 64, 2, 2, 2, 3, 2),
     {"skinny_m16_slab32", {gemm_skinny_kernel<OUT8, 1, 2>, gemm_skinny_kernel<OUT32, 1, 2>, gemm_skinny_kernel<OUT16, 1, 2>}, 16, 32, 64, 512, true, true},
+    {"rows4_m16", {gemm_rows4_kernel<OUT8>, gemm_rows4_kernel<OUT32>, gemm_rows4_kernel<OUT16>}, 16, 4, 1024, (R4_NW + 1) * 64, true, false, 0, true},
 };
 static const int g_num_configs = (int)(sizeof(g_configs) / sizeof(g_configs[0]));
 
@@ -1481,7 +1645,9 @@ static bool stream_eligible(const GemmParams& p) {
 static int pick_config(const GemmParams& p) {
   if (!fast_eligible(p)) return CFG_GATHER;
   if (p.M <= 16) {
-    // two slabs per wave halve the A re-reads; worth it only while enough waves remain (measured)
+    // one GEMM over a long K: stream the weights as whole row pieces; short K or batched (the
+    // decode attention BMMs): MFMA-layout loads, two slabs per wave while enough waves remain
+    if (p.batch == 1 && p.K >= 1024) return CFG_ROWS4_16;
     return (p.N + 31) / 32 >= 160 ? CFG_SKINNY_16_G2 : CFG_SKINNY_16;
   }
   if (p.M <= 64) return CFG_SKINNY_16 + (p.M > 16) + (p.M > 32);
@@ -1572,9 +1738,21 @@ static int run(GemmParams p, int config, hipStream_t stream) {
   if (config < 0) config = (trunc8 && p.M > 64) ? CFG_GATHER : pick_config(p);
   if (config >= g_num_configs) return fail(TI_E_COMBO, "config %d out of range", config);
   const Config& k = g_configs[config];
-  if (k.fast && !k.skinny && trunc8) return fail(TI_E_COMBO, "config %s does not implement TI_ROUND_TRUNC for int8 outputs", k.name);
+  if (k.fast && !k.skinny && !k.rows4 && trunc8) return fail(TI_E_COMBO, "config %s does not implement TI_ROUND_TRUNC for int8 outputs", k.name);
   if (k.fast && !fast_eligible(p)) return fail(TI_E_COMBO, "config %s needs K-contiguous 16-byte aligned operands", k.name);
   if (k.stream_occ && !stream_eligible(p)) return fail(TI_E_COMBO, "config %s needs a row-major output with 16-byte aligned rows", k.name);
+  if (k.rows4) {
+    if (p.M > k.bm) return fail(TI_E_COMBO, "config %s needs M <= %d", k.name, k.bm);
+    // few weight rows: two waves per unit (even / odd chunks of K), so that every wave streams
+    const int units = (p.N + R4_RG - 1) / R4_RG;
+    p.ksplit = (units <= 1024 && p.K > R4_KC) ? 2 : 1;
+    const int slots = R4_NW / p.ksplit;
+    int blocks = (units + slots - 1) / slots;
+    if (blocks > 256) blocks = 256;
+    g_last_config = config;
+    k.fn[out_class(p.out_dtype)]<<<dim3((unsigned)blocks, (unsigned)p.batch), dim3(k.threads), 0, stream>>>(p);
+    return launch_status(k.name);
+  }
   if (k.skinny) {
     if (p.M > k.bm) return fail(TI_E_COMBO, "config %s needs M <= %d", k.name, k.bm);
     // a wave owns one group of k.bn rows of B; split K between the waves of a workgroup while
