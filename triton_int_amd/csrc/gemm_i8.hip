@@ -1746,9 +1746,11 @@ static int run(GemmParams p, int config, hipStream_t stream) {
     // few weight rows: two waves per unit (even / odd chunks of K), so that every wave streams
     const int units = (p.N + R4_RG - 1) / R4_RG;
     p.ksplit = (units <= 1024 && p.K > R4_KC) ? 2 : 1;
+    // every wave of a workgroup gets the same number of units (they meet at a barrier per chunk
+    // of K), and the workgroups fit the chip in one round
     const int slots = R4_NW / p.ksplit;
-    int blocks = (units + slots - 1) / slots;
-    if (blocks > 256) blocks = 256;
+    const int per = slots * ((units + slots * 256 - 1) / (slots * 256));
+    const int blocks = (units + per - 1) / per;
     g_last_config = config;
     k.fn[out_class(p.out_dtype)]<<<dim3((unsigned)blocks, (unsigned)p.batch), dim3(k.threads), 0, stream>>>(p);
     return launch_status(k.name);
