@@ -124,19 +124,51 @@ def mfma_issue_peak(torch, lib, random_operands):
     return ops.value / (s.elapsed_time(e) * 1e-3) / 1e12
 
 
+def _find_sclk_file(torch, glob):
+    """pp_dpm_sclk of the GPU torch uses (matched by PCI address), or of the only AMD GPU in sysfs."""
+    cands = sorted(glob.glob("/sys/bus/pci/devices/*/pp_dpm_sclk"))
+    try:
+        pr = torch.cuda.get_device_properties(0)
+        addr = f"{pr.pci_domain_id:04x}:{pr.pci_bus_id:02x}:{pr.pci_device_id:02x}.0"
+        for c in cands:
+            if addr in c:
+                return c
+    except Exception:
+        pass
+    return cands[0] if len(cands) == 1 else None
+
+
+def _read_sclk_mhz(path):
+    """Current shader clock: the line of pp_dpm_sclk marked with '*'."""
+    import re
+
+    if not path:
+        return None
+    try:
+        with open(path) as f:
+            for line in f:
+                if "*" in line:
+                    m = re.search(r"(\d+)\s*Mhz", line, re.I)
+                    return int(m.group(1)) if m else None
+    except OSError:
+        return None
+    return None
+
+
 def sustained_clock(torch, dev, seconds=2.5):
-    """fc2-shaped GEMM (2048 x 4096 x 16384, fp32 out) looped for `seconds` while rocm-smi is sampled
-    from a thread: sustained TOPS and the shader clock the chip holds under that load, once with
+    """fc2-shaped GEMM (2048 x 4096 x 16384, fp32 out) looped for `seconds` while the driver's
+    pp_dpm_sclk file is sampled from a thread: sustained TOPS and the shader clock the chip holds under that load, once with
     uniform random int8 operands and once with all-zero operands (same instruction stream, no
     operand toggling).  The difference is the power limit, not the kernel."""
+    import glob
     import re
-    import subprocess
     import threading
 
     from triton_int_amd.kernels import linear
 
     M, N, K = 2048, 4096, 16384
     out = {}
+    sclk_file = _find_sclk_file(torch, glob)
     for kind in ("uniform", "zeros"):
         if kind == "uniform":
             ws = [torch.randint(-127, 128, (N, K), dtype=torch.int8, device=dev) for _ in range(8)]
@@ -148,15 +180,12 @@ def sustained_clock(torch, dev, seconds=2.5):
         clocks = []
 
         def sample():
+            # the driver's sysfs file, read in-process (no child process is started once the GPU is in use)
             for _ in range(int(seconds / 0.5)):
                 time.sleep(0.4)
-                try:
-                    r = subprocess.run(["/opt/rocm/bin/rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=5)
-                    m = re.search(r"sclk clock level:[^(]*\((\d+)Mhz\)", r.stdout)
-                    if m:
-                        clocks.append(int(m.group(1)))
-                except Exception:
-                    pass
+                mhz = _read_sclk_mhz(sclk_file)
+                if mhz:
+                    clocks.append(mhz)
 
         th = threading.Thread(target=sample)
         th.start()
