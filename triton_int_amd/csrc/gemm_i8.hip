@@ -3,11 +3,16 @@
 // Replaces the Triton kernels of zhanglei1172/triton_int kernels/linear.py:24-853,
 // kernels/bmm.py:12-760 and kernels/fused.py:88-231 (one tl.dot K loop + per-kernel epilogue).
 //
-// Two kernel families:
-//   gemm_mfma_kernel   both operands K-contiguous and 16-byte aligned.  128-bit buffer loads
-//                      (optionally straight into LDS), XOR-swizzled LDS tiles, double buffering,
-//                      v_mfma_i32_32x32x32_i8 with a 64-lane wavefront owning a WTM x WTN sub-tile.
-//   gemm_gather_kernel any strides / alignment / K (byte gathers); same MFMA and epilogue.
+// Kernels (all v_mfma_i32_*_i8, int32 accumulators in registers):
+//   gemm_mfma_ws_kernel      persistent, wave-specialised: producer waves issue the global -> LDS
+//                            loads, consumer waves read fragments and issue MFMAs.  The large GEMMs.
+//   gemm_mfma_stream_kernel  persistent, loads issued by the MFMA waves (256x256 tiles, short K).
+//   gemm_mfma_kernel         one tile per workgroup; any output layout the fast loads allow.
+//   gemm_rows4_kernel        M <= 16: weights streamed as whole 1 KB row pieces (decode linears).
+//   gemm_skinny_kernel       M <= 64: 16-row weight slabs in MFMA layout, K split over waves.
+//   gemm_gather_kernel       any strides / alignment / K (byte gathers).
+// The first five need both operands K-contiguous and 16-byte aligned: 128-bit buffer loads
+// straight into XOR-swizzled LDS tiles, several stages deep.
 //
 // C = epilogue(sum_k A[m,k] * B[n,k]); A is [M,K], B is [N,K] (the reference's "N" operand,
 // kernels/linear.py:217), the "T" operand [K,N] arrives as strides (sBn = 1, sBk = N).
