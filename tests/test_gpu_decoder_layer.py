@@ -110,3 +110,34 @@ def test_decoder_layer_opt13b_shapes_run():
     assert np.array_equal(cpu(tr["scores"]), O.bmm_s8t_s8n_s8t(cpu(tr["q"]), cpu(tr["k_all"]), np.float32(layer.qk_alpha)))
     acc = O.linear_a8_w8_b32_o32(cpu(tr["ctx"])[0], cpu(layer.out_proj.weight), cpu(layer.out_proj.bias))
     assert np.array_equal(cpu(tr["acc"])[0], acc)
+
+
+def test_layer_replayed_from_a_hip_graph_matches_eager():
+    """The decode pass and a small prefill pass captured into a HIP graph: every replay (with the
+    program's own eager launches and synchronisations in between) must reproduce the eager output
+    bit for bit — the kernels keep no state between launches and the library records no memsets."""
+    from triton_int_amd.nn.opt import W8A8OPTDecoderLayer
+
+    layer = W8A8OPTDecoderLayer(hidden=1024, heads=8, ffn=4096).randomize(seed=5).to(DEV)
+    g = torch.Generator(device="cpu").manual_seed(11)
+    for S, T in ((16, 272), (192, 192)):
+        x = torch.randn((1, S, 1024), generator=g).to(DEV)
+        kc0 = torch.randint(-127, 128, (8, T, 128), dtype=torch.int8, generator=g).to(DEV)
+        vc0 = torch.randint(-127, 128, (8, 128, T), dtype=torch.int8, generator=g).to(DEV)
+        want = layer(x, kv_cache=(kc0.clone(), vc0.clone())).clone()
+        kc, vc = kc0.clone(), vc0.clone()
+        graph, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            layer(x, kv_cache=(kc, vc))  # warm-up on the capture stream (allocator, scale cache)
+            torch.cuda.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                out = layer(x, kv_cache=(kc, vc))
+        torch.cuda.synchronize()
+        for rep in range(3):
+            out.zero_()
+            kc.copy_(kc0); vc.copy_(vc0)
+            layer(torch.randn_like(x))  # unrelated eager work between replays
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, want), f"S={S} replay {rep}"
