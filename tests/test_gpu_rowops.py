@@ -154,7 +154,7 @@ def test_gelu_q_grid_and_module():
     assert mx <= 1 and rate < 1e-3
 
 
-@pytest.mark.parametrize("rows,cols,q_len", [(64, 2048, 0), (48, 2048, 16), (10, 300, 5), (7, 17, 0), (6, 4096, 3), (4, 8192, 0), (5, 1, 0)])
+@pytest.mark.parametrize("rows,cols,q_len", [(64, 2048, 0), (48, 2048, 16), (10, 300, 5), (7, 17, 0), (6, 4096, 3), (4, 8192, 0), (5, 1, 0), (9, 1040, 3), (12, 1536, 12)])
 def test_softmax_q(rows, cols, q_len):
     fused = _fused()
     g = rng(rows + cols)
@@ -168,6 +168,10 @@ def test_softmax_q(rows, cols, q_len):
         assert got.min() >= 0
     x3 = x.reshape(1, rows, cols)
     assert fused.softmax_q(gpu(x3), 0.05).shape == (1, rows, cols)
+    # scale 0 (every unmasked column equally likely) goes through the general kernel
+    got = cpu(fused.softmax_q(gpu(x), 0.0, causal_q_len=q_len))
+    mx, rate = mismatch_report(got, O.softmax_q(x, 0.0, causal_q_len=q_len))
+    assert mx <= 1
 
 
 @pytest.mark.parametrize("rows,cols", [(2048, 5120), (16, 5120), (1, 128), (70, 33), (64, 64), (129, 257)])

@@ -262,13 +262,94 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// Rows whose start and length are multiples of 16 bytes.  Every load of a row is issued before the
+// first use: buffer loads whose offset is pushed out of range for chunks beyond the causal limit
+// (they return 0 without touching memory), then masking in registers.  Stores are range-checked
+// buffer stores, so neither phase branches around a memory instruction.
+template <int VPT>
+__global__ __launch_bounds__(SM_WAVES * 64) void softmax_q_kernel(const int8_t* __restrict__ x, int64_t x_rs,
+                                                                  float scale, int8_t* __restrict__ y, int64_t y_rs,
+                                                                  int rows, int cols, int causal_q_len) {
+  const int lane = threadIdx.x & 63;
+  const int row = __builtin_amdgcn_readfirstlane(blockIdx.x * SM_WAVES + (threadIdx.x >> 6));
+  if (row >= rows) return;
+  const int limit = causal_q_len > 0 ? min(cols, (row % causal_q_len) + (cols - causal_q_len) + 1) : cols;
+  const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc((void*)(x + (int64_t)row * x_rs), 0, cols, 0x00020000);
+  const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc((void*)(y + (int64_t)row * y_rs), 0, cols, 0x00020000);
+  // masked elements are -inf: they drop out of the maximum, and with scale > 0 their exponential
+  // is exactly 0, so neither the sum nor the output phase has to look at the mask again
+  const float NEG = -__builtin_inff();
+  const int OOB = 0x7ffffff0;
+
+  v4i w[VPT];
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int c0 = (j * 64 + lane) * 16;
+    w[j] = __builtin_amdgcn_raw_buffer_load_b128(rx, c0 < limit ? c0 : OOB, 0, 2);
+  }
+  float f[VPT][16];
+  float mx = NEG;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int c0 = (j * 64 + lane) * 16;
+    if (c0 >= limit) continue;  // whole 1 KB pieces beyond the limit cost no VALU work
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const unsigned u = (unsigned)w[j][g] ^ 0x80808080u;
+      // the compiler turns these into v_cvt_f32_ubyte0..3
+      f[j][4 * g + 0] = (float)(u & 0xffu);
+      f[j][4 * g + 1] = (float)((u >> 8) & 0xffu);
+      f[j][4 * g + 2] = (float)((u >> 16) & 0xffu);
+      f[j][4 * g + 3] = (float)(u >> 24);
+    }
+    if (c0 + 16 > limit) {  // the chunk that straddles the limit
+#pragma unroll
+      for (int t = 0; t < 16; ++t) f[j][t] = c0 + t < limit ? f[j][t] : NEG;
+    }
+#pragma unroll
+    for (int t = 0; t < 16; t += 2) mx = fmaxf(fmaxf(mx, f[j][t]), f[j][t + 1]);  // v_max3_f32
+  }
+  mx = wave_max(mx);
+  const float s2 = scale * 1.44269504088896340736f;  // exp(v) = exp2(v * log2 e)
+  const float c = -(mx * s2);
+  float sum = 0.0f;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int c0 = (j * 64 + lane) * 16;
+    if (c0 >= limit) continue;
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+      f[j][t] = __builtin_amdgcn_exp2f(__builtin_fmaf(f[j][t], s2, c));
+      sum += f[j][t];
+    }
+  }
+  sum = wave_sum(sum);
+  const float r = 127.0f / sum;
+#pragma unroll
+  for (int j = 0; j < VPT; ++j) {
+    const int c0 = (j * 64 + lane) * 16;
+    v4i o = {0, 0, 0, 0};
+    if (c0 < limit) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const unsigned b0 = __float_as_uint(__builtin_fmaf(f[j][4 * g + 0], r, 12582912.0f));
+        const unsigned b1 = __float_as_uint(__builtin_fmaf(f[j][4 * g + 1], r, 12582912.0f));
+        const unsigned b2 = __float_as_uint(__builtin_fmaf(f[j][4 * g + 2], r, 12582912.0f));
+        const unsigned b3 = __float_as_uint(__builtin_fmaf(f[j][4 * g + 3], r, 12582912.0f));
+        o[g] = (int)(__builtin_amdgcn_perm(b1, b0, 0x0c0c0400u) | __builtin_amdgcn_perm(b3, b2, 0x04000c0cu));
+      }
+    }
+    __builtin_amdgcn_raw_buffer_store_b128(o, ry, c0, 0, 2);  // dropped beyond the row's end
+  }
+}
+
 // Per element the work is: byte -> float (v_cvt_f32_ubyteN on the sign-flipped dword, so the float
 // is x + 128), one fma that forms (x - max) * scale * log2(e), the hardware exp2, one add for the
 // sum; then one fma e * (127 / sum) + 1.5 * 2^23, whose low byte is the rounded probability (it
 // lies in [0, 127], no clamp), and byte permutes to pack.  16-byte chunks that lie wholly beyond a
 // causal limit are neither read nor computed, the one chunk that straddles it is masked.
 template <int VPT>
-__global__ __launch_bounds__(SM_WAVES * 64) void softmax_q_kernel(const int8_t* __restrict__ x, int64_t x_rs,
+__global__ __launch_bounds__(SM_WAVES * 64) void softmax_q_any_kernel(const int8_t* __restrict__ x, int64_t x_rs,
                                                                   float scale, int8_t* __restrict__ y, int64_t y_rs,
                                                                   int rows, int cols, int causal_q_len) {
   const int lane = threadIdx.x & 63;
@@ -289,7 +370,9 @@ __global__ __launch_bounds__(SM_WAVES * 64) void softmax_q_kernel(const int8_t* 
     if (c0 >= limit) {
 #pragma unroll
       for (int t = 0; t < 16; ++t) f[j][t] = NEG;
-    } else if (vec && c0 + 16 <= limit) {
+    } else if (vec && c0 + 16 <= cols) {
+      // a chunk that straddles the causal limit is still inside the row: load it whole and mask
+      // in registers, so that no wave waits for a second, dependent round of byte loads
       v4u w = __builtin_nontemporal_load((const v4u*)(xr + c0));
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
@@ -299,6 +382,10 @@ __global__ __launch_bounds__(SM_WAVES * 64) void softmax_q_kernel(const int8_t* 
         f[j][4 * g + 1] = (float)((u >> 8) & 0xffu);
         f[j][4 * g + 2] = (float)((u >> 16) & 0xffu);
         f[j][4 * g + 3] = (float)(u >> 24);
+      }
+      if (c0 + 16 > limit) {
+#pragma unroll
+        for (int t = 0; t < 16; ++t) f[j][t] = c0 + t < limit ? f[j][t] : NEG;
       }
 #pragma unroll
       for (int t = 0; t < 16; t += 2) mx = fmaxf(fmaxf(mx, f[j][t]), f[j][t + 1]);  // v_max3_f32
@@ -318,20 +405,14 @@ __global__ __launch_bounds__(SM_WAVES * 64) void softmax_q_kernel(const int8_t* 
   for (int j = 0; j < VPT; ++j) {
     const int c0 = (j * 64 + lane) * 16;
     if (c0 >= limit) continue;
-    if (c0 + 16 <= limit) {
 #pragma unroll
-      for (int t = 0; t < 16; ++t) {
-        f[j][t] = __builtin_amdgcn_exp2f(__builtin_fmaf(f[j][t], s2, c));
-        sum += f[j][t];
-      }
-    } else {  // the chunk that straddles the limit (or the end of the row)
+    for (int t = 0; t < 16; ++t) f[j][t] = __builtin_amdgcn_exp2f(__builtin_fmaf(f[j][t], s2, c));
+    if (c0 + 16 > limit) {  // the chunk that straddles the limit (or the end of the row)
 #pragma unroll
-      for (int t = 0; t < 16; ++t) {
-        const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(f[j][t], s2, c));
-        f[j][t] = f[j][t] < 0.0f ? 0.0f : e;
-        sum += f[j][t];
-      }
+      for (int t = 0; t < 16; ++t) f[j][t] = c0 + t < limit ? f[j][t] : 0.0f;
     }
+#pragma unroll
+    for (int t = 0; t < 16; ++t) sum += f[j][t];
   }
   sum = wave_sum(sum);
   const float r = 127.0f / sum;
@@ -497,10 +578,17 @@ int ti_softmax_q(const int8_t* x, int64_t x_row_stride, float scale, int8_t* y, 
   hipStream_t s = (hipStream_t)stream;
   dim3 grid((unsigned)((rows + ti::SM_WAVES - 1) / ti::SM_WAVES)), block(ti::SM_WAVES * 64);
   const int vpt = (cols + 1023) / 1024;
-  if (vpt <= 1) ti::softmax_q_kernel<1><<<grid, block, 0, s>>>(x, x_row_stride, scale, y, y_row_stride, rows, cols, causal_q_len);
-  else if (vpt <= 2) ti::softmax_q_kernel<2><<<grid, block, 0, s>>>(x, x_row_stride, scale, y, y_row_stride, rows, cols, causal_q_len);
-  else if (vpt <= 4) ti::softmax_q_kernel<4><<<grid, block, 0, s>>>(x, x_row_stride, scale, y, y_row_stride, rows, cols, causal_q_len);
-  else ti::softmax_q_kernel<8><<<grid, block, 0, s>>>(x, x_row_stride, scale, y, y_row_stride, rows, cols, causal_q_len);
+  const bool aligned = ((((uintptr_t)x) | ((uintptr_t)y) | (uintptr_t)x_row_stride | (uintptr_t)y_row_stride | (uintptr_t)cols) & 15) == 0;
+#define TI_SOFTMAX_LAUNCH(KERNEL)                                                                          \
+  do {                                                                                                     \
+    if (vpt <= 1) KERNEL<1><<<grid, block, 0, s>>>(x, x_row_stride, scale, y, y_row_stride, rows, cols, causal_q_len);      \
+    else if (vpt <= 2) KERNEL<2><<<grid, block, 0, s>>>(x, x_row_stride, scale, y, y_row_stride, rows, cols, causal_q_len); \
+    else if (vpt <= 4) KERNEL<4><<<grid, block, 0, s>>>(x, x_row_stride, scale, y, y_row_stride, rows, cols, causal_q_len); \
+    else KERNEL<8><<<grid, block, 0, s>>>(x, x_row_stride, scale, y, y_row_stride, rows, cols, causal_q_len);               \
+  } while (0)
+  if (aligned && scale > 0.0f) TI_SOFTMAX_LAUNCH(ti::softmax_q_kernel);
+  else TI_SOFTMAX_LAUNCH(ti::softmax_q_any_kernel);
+#undef TI_SOFTMAX_LAUNCH
   return ti::launch_status("softmax_q_kernel");
 }
 
