@@ -533,6 +533,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
 #ifndef TI_STREAM_STORE_AUX
 #define TI_STREAM_STORE_AUX 2  // nt: the outputs are streamed, keep the operand panels in L2
 #endif
+// bytes of the per-wave LDS strip of the int8 epilogue: 32 rows of the wave's WTN output bytes when
+// WTN / 16 is a power of two (the swizzle below needs that), none otherwise (direct stores)
+constexpr int epi_strip_bytes(int wtn) { return ((wtn / 16) & (wtn / 16 - 1)) == 0 ? 32 * wtn : 0; }
+
 template <int TM, int TN, int OUTCLS>
 __device__ __forceinline__ void stream_epilogue(const GemmParams& p, const EpiCtx& e, v16i (&acc)[TM][TN], int bz,
                                                 int mw, int nw, char* strip, int lane) {
@@ -557,9 +561,10 @@ __device__ __forceinline__ void stream_epilogue(const GemmParams& p, const EpiCt
     // strip row r lives at slot s ^ ((r / WRAP) % SEG), WRAP = rows per 256 bytes: conflict-free
     // for the column-wise writes and the row-wise reads.  The area is private to the wave: no
     // barrier, LDS operations of one wave execute in order.
-    constexpr int SEG = WTN / 16, RP = 64 / SEG, WRAP = 256 / WTN;
-    static_assert(32 % RP == 0 && 32 / RP == TN, "one read pass per 32-column block");
-    float* cols = (float*)(strip + 32 * WTN);
+    constexpr bool VIA_STRIP = epi_strip_bytes(WTN) != 0;
+    constexpr int SEG = WTN / 16, RP = VIA_STRIP ? 64 / SEG : 1, WRAP = VIA_STRIP ? 256 / WTN : 1;
+    static_assert(!VIA_STRIP || (32 % RP == 0 && 32 / RP == TN), "one read pass per 32-column block");
+    float* cols = (float*)(strip + epi_strip_bytes(WTN));
     const float q_floor = e.epilogue == TI_EPI_SCALE_RELU_I8 ? 0.0f : -128.0f;
     const int w_swz = (lrow / WRAP) & (SEG - 1);
     const int r_row = lane / SEG, r_seg = lane % SEG;
@@ -597,16 +602,27 @@ __device__ __forceinline__ void stream_epilogue(const GemmParams& p, const EpiCt
           const auto s13 = __builtin_amdgcn_permlane32_swap(X[1], X[3], false, false);
           v4u v;
           v[0] = s02[0]; v[1] = s02[1]; v[2] = s13[0]; v[3] = s13[1];
-          *(v4u*)(strip + lrow * WTN + (((2 * j + lhi) ^ w_swz) * 16)) = v;
+          if constexpr (VIA_STRIP) {
+            *(v4u*)(strip + lrow * WTN + (((2 * j + lhi) ^ w_swz) * 16)) = v;
+          } else {
+            // no strip for this tile width: the lane stores its 16 bytes of row lrow itself (an
+            // instruction touches 32 rows with 32 bytes each; left to L2 to merge into lines)
+            const int m = mw + i * 32 + lrow;
+            const int n = nw + (2 * j + lhi) * 16;
+            const int off = (m < p.M && n < p.N) ? m * ldc + n : OOB;
+            __builtin_amdgcn_raw_buffer_store_b128(v, rC, off, 0, 0);
+          }
         }
+        if constexpr (VIA_STRIP) {
 #pragma unroll
-        for (int q = 0; q < TN; ++q) {
-          const int row = q * RP + r_row;
-          const v4u v = *(const v4u*)(strip + row * WTN + ((r_seg ^ ((row / WRAP) & (SEG - 1))) * 16));
-          const int m = mw + i * 32 + row;
-          const int n = nw + r_seg * 16;
-          const int off = (m < p.M && n < p.N) ? m * ldc + n : OOB;  // N % 16 == 0: a segment is in or out
-          __builtin_amdgcn_raw_buffer_store_b128(v, rC, off, 0, TI_STREAM_STORE_AUX);
+          for (int q = 0; q < TN; ++q) {
+            const int row = q * RP + r_row;
+            const v4u v = *(const v4u*)(strip + row * WTN + ((r_seg ^ ((row / WRAP) & (SEG - 1))) * 16));
+            const int m = mw + i * 32 + row;
+            const int n = nw + r_seg * 16;
+            const int off = (m < p.M && n < p.N) ? m * ldc + n : OOB;  // N % 16 == 0: a segment is in or out
+            __builtin_amdgcn_raw_buffer_store_b128(v, rC, off, 0, TI_STREAM_STORE_AUX);
+          }
         }
       }
     };
@@ -695,7 +711,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
   constexpr int STAGE = A_BYTES + B_BYTES;
   // int8 outputs: per wave a 32-row strip of its WTN output bytes (to turn the MFMA layout into
   // long row segments) and WTN per-column fp32 terms
-  constexpr int STRIP = 32 * WTN, COLS = 4 * WTN;
+  constexpr int STRIP = epi_strip_bytes(WTN), COLS = 4 * WTN;
   constexpr int EPI_LDS = OUTCLS == OUT8 ? WAVES_M * WAVES_N * (STRIP + COLS) : 0;
   constexpr int LDS_BYTES = NSTAGE * STAGE + EPI_LDS;
   constexpr int DEPTH = NSTAGE - 1;
@@ -936,7 +952,7 @@ __global__ __launch_bounds__((WAVES_M * WAVES_N + PW) * 64) void gemm_mfma_ws_ke
   constexpr int KS = BK / 32;
   constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK;
   constexpr int STAGE = A_BYTES + B_BYTES;
-  constexpr int STRIP = 32 * WTN, COLS = 4 * WTN;
+  constexpr int STRIP = epi_strip_bytes(WTN), COLS = 4 * WTN;
   constexpr int EPI_LDS = OUTCLS == OUT8 ? NWC * (STRIP + COLS) : 0;
   constexpr int LDS_BYTES = NSTAGE * STAGE + EPI_LDS;
   constexpr int DEPTH = NSTAGE - 1;
@@ -1586,6 +1602,7 @@ enum ConfigId {
   CFG_STREAM_128x128,
   CFG_SKINNY_16_G2,  // M <= 16, a wave owns 2 slabs that share its A fragments
   CFG_ROWS4_16,      // M <= 16, K >= 1024: weights streamed as 1 KB row pieces
+  CFG_WS_256x160,    // 2048 x 5120 outputs are exactly 256 of these tiles: one full round of the chip
 };
 
 static const Config g_configs[] = {
@@ -1602,6 +1619,7 @@ static const Config g_configs[] = {
     TI_STREAM(128, 128, 64, 2, 2, 2, 3, 2),
     {"skinny_m16_slab32", {gemm_skinny_kernel<OUT8, 1, 2>, gemm_skinny_kernel<OUT32, 1, 2>, gemm_skinny_kernel<OUT16, 1, 2>}, 16, 32, 64, 512, true, true},
     {"rows4_m16", {gemm_rows4_kernel<OUT8>, gemm_rows4_kernel<OUT32>, gemm_rows4_kernel<OUT16>}, 16, 4, 1024, (R4_NW + 1) * 64, true, false, 0, true},
+    TI_WS(256, 160, 128, 4, 1, 1, 3, 4),
 };
 static const int g_num_configs = (int)(sizeof(g_configs) / sizeof(g_configs[0]));
 
@@ -1665,10 +1683,12 @@ static int pick_config(const GemmParams& p) {
       {stream ? CFG_WS_256x128 : CFG_TILE_256x128, stream ? 1.00 : 0.90},
       {stream ? CFG_STREAM_128x128 : CFG_TILE_128x128, 0.78},
       {CFG_TILE_64x64, 0.50},
+      {stream ? CFG_WS_256x160 : -1, 1.00},
   };
   int best = CFG_TILE_64x64;
   double best_score = -1.0;
   for (const Cand& c : cands) {
+    if (c.cfg < 0) continue;
     const Config& k = g_configs[c.cfg];
     const int slots = 256 * (k.stream_occ > 1 ? k.stream_occ : 1);
     const int64_t tm = (p.M + k.bm - 1) / k.bm, tn = (p.N + k.bn - 1) / k.bn;
@@ -1743,6 +1763,7 @@ static int run(GemmParams p, int config, hipStream_t stream) {
   if (config < 0) config = (trunc8 && p.M > 64) ? CFG_GATHER : pick_config(p);
   if (config >= g_num_configs) return fail(TI_E_COMBO, "config %d out of range", config);
   const Config& k = g_configs[config];
+  if (!k.fn[out_class(p.out_dtype)]) return fail(TI_E_COMBO, "config %s has no kernel for output dtype %d", k.name, p.out_dtype);
   if (k.fast && !k.skinny && !k.rows4 && trunc8) return fail(TI_E_COMBO, "config %s does not implement TI_ROUND_TRUNC for int8 outputs", k.name);
   if (k.fast && !fast_eligible(p)) return fail(TI_E_COMBO, "config %s needs K-contiguous 16-byte aligned operands", k.name);
   if (k.stream_occ && !stream_eligible(p)) return fail(TI_E_COMBO, "config %s needs a row-major output with 16-byte aligned rows", k.name);
