@@ -292,34 +292,31 @@ def decoder_layer_ms(torch, dev):
         layers[state["i"]](x)
 
     out = {"prefill_1x2048_ms": time_region(torch, prefill, 10, 2)}
-    # per-op breakdown of the prefill: each stage on the tensors a traced forward produced, timed alone
-    from triton_int_amd.kernels.bmm import bmm_s8t_s8n_s8t
-    from triton_int_amd.kernels.fused import softmax_q
+    # per-stage breakdown of the prefill, in sequence: stream events between the stages of the same
+    # alternating forward passes (weights cold, clocks as the whole layer holds them)
+    reps, marks = 8, []
 
-    tr, L0 = {}, layers[0]
-    L0(x, _trace=tr)
-    ctx_v = torch.empty_like(tr["ctx"])
-    stages = {
-        "ln1_layernorm_q": lambda: L0.ln1(x),
-        "qkv_3x_linear_o8": lambda: (L0.q_proj(tr["h8"]), L0.k_proj(tr["h8"]), L0.v_proj(tr["h8"])),
-        "qk_bmm_o8": lambda: bmm_s8t_s8n_s8t(tr["q"], tr["k_all"], L0.qk_alpha, out=tr["scores"]),
-        "softmax_q_causal": lambda: softmax_q(tr["scores"], L0.score_scale, causal_q_len=2048),
-        "pv_bmm_o8": lambda: bmm_s8t_s8n_s8t(tr["probs"], tr["vt_all"], L0.pv_alpha,
-                                             out=ctx_v[0].view(2048, 40, 128).transpose(0, 1)),
-        "out_proj_linear_o32": lambda: L0.out_proj(tr["ctx"]),
-        "ln2_dq_add_layernorm_q": lambda: L0.ln2(x, tr["acc"]),
-        "fc1_linear_gelu_q": lambda: L0.fc1(tr["h8b"]),
-        "fc2_linear_f32": lambda: L0.fc2(tr["f8"]),
-    }
-    br = {k: time_region(torch, f, 10, 2) for k, f in stages.items()}
-    br["glue_head_split_transpose_residual_add"] = max(0.0, out["prefill_1x2048_ms"] - sum(br.values()))
+    def mark(name):
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record()
+        marks.append((name, ev))
+
+    for _ in range(reps):
+        state["i"] ^= 1
+        mark("start")
+        layers[state["i"]](x, _mark=mark)
+    torch.cuda.synchronize()
+    br = {}
+    for (n0, e0), (n1, e1) in zip(marks, marks[1:]):
+        if n1 != "start":
+            br[n1] = br.get(n1, 0.0) + e0.elapsed_time(e1) / reps
     out["prefill_breakdown_ms"] = br
+    out["prefill_breakdown_sum_ms"] = sum(br.values())
     # ideal: GEMM/BMM ops at the 5.0 POP/s peak, row kernels at 8 TB/s on their algorithmic bytes
     S_, H_, F_ = 2048, 5120, 20480
     ideal = 1374.4e9 / 5.0e15 + (S_ * H_ * 5 + S_ * H_ * 13 + 40 * S_ * S_ * 2) / 8.0e12
     out["prefill_ideal_ms"] = ideal * 1e3
     out["prefill_ideal_over_measured"] = ideal * 1e3 / out["prefill_1x2048_ms"]
-    del tr, ctx_v
     kc = torch.randint(-127, 128, (40, 2048, 128), dtype=torch.int8, device=dev)
     vc = torch.randint(-127, 128, (40, 128, 2048), dtype=torch.int8, device=dev)
     xd = torch.randn((1, 16, 5120), device=dev)

@@ -129,6 +129,24 @@ int ti_bmm_i8_config(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk,
                      const float* alpha, const float* beta,
                      int epilogue, int out_dtype, int round_mode,
                      int config, void* stream);
+/*
+ * Grouped form: the batches are different projections rather than slices of one operand.  Batch b
+ * adds bias elements [b * bias_batch_stride, b * bias_batch_stride + N) and scales with
+ * alpha[b * scale_batch_stride], beta[b * scale_batch_stride]; everything else is ti_bmm_i8_config.
+ * With sAb = 0 (one shared activation matrix), B = the projections' [N,K] weights stacked along N
+ * (sBb = N * sBn) and sCb = N (batch b writes columns b*N .. of a [M, batch*N] row-major output)
+ * this is the q/k/v projection of an attention block as one launch: each projection alone is
+ * too small to fill the chip (W8A8B8O8Linear x3, nn/linear.py:18-67; the reference launches them
+ * one by one).  No counterpart in the reference's kernels.
+ */
+int ti_bmm_i8_grouped(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk,
+                      const int8_t* B, int64_t sBb, int64_t sBn, int64_t sBk,
+                      void* C, int64_t sCb, int64_t sCm, int64_t sCn,
+                      int batch, int M, int N, int K,
+                      const void* bias, int bias_kind, int64_t bias_batch_stride,
+                      const float* alpha, const float* beta, int64_t scale_batch_stride,
+                      int epilogue, int out_dtype, int round_mode,
+                      int config, void* stream);
 int ti_gemm_num_configs(void);
 const char* ti_gemm_config_name(int config);
 /* Index of the configuration the calling thread's most recent ti_bmm_i8* launch used (-1 if

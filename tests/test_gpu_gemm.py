@@ -80,6 +80,34 @@ def test_all_configs_int8_epilogues_bit_exact(shape):
         assert np.abs(want_tr.astype(int) - want.astype(int)).max() <= 1
 
 
+@pytest.mark.parametrize("shape", [(300, 272, 384), (16, 1280, 2048), (7, 48, 64), (520, 320, 1040)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_grouped_linear_equals_separate_linears(shape):
+    """Three projections of one input as one launch (per-projection bias rows and scales): every
+    configuration must give, per projection, exactly the single linear's int8 result."""
+    linear, _, _ = _kl()
+    M, N, K = shape
+    g = rng(M * 5 + N)
+    G = 3
+    a = rand_i8(g, M, K)
+    w, bias = rand_i8(g, G * N, K), rand_i8(g, G * N)
+    std = np.sqrt(K) * 127 * 127 / 3
+    alphas = np.array([0.0021, 40.0 / std, 0.5], dtype=np.float32)
+    betas = np.array([0.013, 0.11, 1.0], dtype=np.float32)
+    want = np.concatenate([O.linear_a8_w8_b8_o8(a, w[i * N:(i + 1) * N], bias[i * N:(i + 1) * N], alphas[i], betas[i])
+                           for i in range(G)], axis=1)
+    ga, gw, gb, gal, gbe = gpu(a), gpu(w), gpu(bias), gpu(alphas), gpu(betas)
+    ran = set()
+    for cfg, name in [(-1, "auto")] + _configs(M, N, out8=True):
+        got = cpu(linear.linear_group_a8_w8_b8_o8(ga, gw, gb, gal, gbe, G, _config=cfg))
+        assert got.shape == (M, G * N) and np.array_equal(got, want), f"config {name}"
+        ran.add(name.split("_")[0])
+    assert {"gather", "mfma", "stream", "ws"} <= ran
+    # leading dimensions are kept
+    got = cpu(linear.linear_group_a8_w8_b8_o8(ga.view(1, M, K), gw, gb, gal, gbe, G))
+    assert got.shape == (1, M, G * N) and np.array_equal(got[0], want)
+
+
 @pytest.mark.parametrize("shape", SHAPES[:4], ids=lambda s: "x".join(map(str, s)))
 def test_all_configs_float_and_scaled_i32(shape):
     linear, _, _ = _kl()

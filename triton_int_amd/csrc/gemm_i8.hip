@@ -35,6 +35,10 @@ struct GemmParams {
   int epilogue, out_dtype, round_mode;
   int tiles_m, tiles_n, group_m;
   int ksplit;  // skinny kernel: waves of a workgroup that share one 16-row slab and split K
+  // grouped launches (several projections of one input as the batches of one launch): batch b uses
+  // bias elements [b * bias_bs, b * bias_bs + N) and the scalars alpha[b * scale_bs], beta[b * scale_bs]
+  int64_t bias_bs;
+  int64_t scale_bs;
 };
 
 enum OutClass { OUT8 = 0, OUT32 = 1, OUT16 = 2 };
@@ -150,14 +154,16 @@ __device__ __forceinline__ void store_one(const EpiCtx& e, void* C, int64_t off,
   }
 }
 
-__device__ __forceinline__ EpiCtx make_epi(const GemmParams& p) {
+__device__ __forceinline__ EpiCtx make_epi(const GemmParams& p, int bz) {
   EpiCtx e;
-  e.alpha = p.alpha ? *p.alpha : 1.0f;
-  e.beta = p.beta ? *p.beta : 1.0f;
+  const int64_t si = (int64_t)bz * p.scale_bs;
+  e.alpha = p.alpha ? p.alpha[si] : 1.0f;
+  e.beta = p.beta ? p.beta[si] : 1.0f;
   e.epilogue = p.epilogue;
   e.round_mode = p.round_mode;
   e.bias_kind = p.bias ? p.bias_kind : TI_BIAS_NONE;
-  e.bias = p.bias;
+  const int bias_esz = p.bias_kind == TI_BIAS_I8 ? 1 : 4;
+  e.bias = p.bias ? (const void*)((const char*)p.bias + (int64_t)bz * p.bias_bs * bias_esz) : nullptr;
   e.safe = (const float*)p.A;
   return e;
 }
@@ -402,7 +408,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
   // that depends on the epilogue kind is decided once, outside the unrolled part: one uniform
   // branch selects a specialised body, and the remaining run-time options (rounding mode, ReLU,
   // bias present) are folded into branch-free selects.
-  const EpiCtx e = make_epi(p);
+  const EpiCtx e = make_epi(p, bz);
   char* Cb = (char*)p.C;
   const int lrow = lane & 31, lhi = lane >> 5;
   const bool has_bias = e.bias_kind != TI_BIAS_NONE;
@@ -857,8 +863,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
   constexpr int N_STEADY = LOADS * (DEPTH - 2) + LOADS_A;
   constexpr int N_AFTER_STORES = (N_STEADY + STORES > 63) ? 63 : N_STEADY + STORES;
 
-  const EpiCtx e = make_epi(p);
-
   // ---- fill the pipeline
   aim(0);
 #pragma unroll
@@ -873,6 +877,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
   for (int it = 0; it < count; ++it) {
     int bz, m0, n0;
     locate(it, bz, m0, n0);
+    const EpiCtx e = make_epi(p, bz);  // scalar loads, long done when the epilogue needs them
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -1113,13 +1118,12 @@ __global__ __launch_bounds__((WAVES_M * WAVES_N + PW) * 64) void gemm_mfma_ws_ke
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-  const EpiCtx e = make_epi(p);
-
   asm volatile("s_barrier" ::: "memory");  // k-tile 0 is in LDS
   int st = 0;
   for (int it = 0; it < count; ++it) {
     int bz, m0, n0;
     locate(it, bz, m0, n0);
+    const EpiCtx e = make_epi(p, bz);  // scalar loads, long done when the epilogue needs them
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -1195,7 +1199,7 @@ __global__ __launch_bounds__(256) void gemm_gather_kernel(GemmParams p) {
     __syncthreads();
   }
 
-  const EpiCtx e = make_epi(p);
+  const EpiCtx e = make_epi(p, bz);
   constexpr int ESZ = OUTCLS == OUT8 ? 1 : (OUTCLS == OUT32 ? 4 : 2);
   char* Cz = (char*)p.C + (int64_t)bz * p.sCb * ESZ;
   const int n = n0 + wn * 32 + (lane & 31);
@@ -1256,7 +1260,7 @@ __global__ __launch_bounds__(512, UU ? 2 : 4) void gemm_skinny_kernel(GemmParams
 
   // The epilogue's scalars and per-column terms are fetched now, ahead of the weight stream: at the
   // end of the kernel each of them would cost a full memory round trip with nothing to overlap.
-  const EpiCtx e = make_epi(p);
+  const EpiCtx e = make_epi(p, bz);
   float col[G][4];
   int bias_i32[G][4];
 #pragma unroll
@@ -1455,7 +1459,7 @@ __global__ __launch_bounds__((R4_NW + 1) * 64) void gemm_rows4_kernel(GemmParams
   const int r16 = lane & 15, c4 = lane >> 4;
   const int w_lane = (r16 & (R4_RG - 1)) * R4_PITCH + c4 * 16;  // rows 4..15 of the operand repeat rows 0..3
   const int x_lane = r16 * R4_PITCH + c4 * 16;
-  const EpiCtx e = make_epi(p);
+  const EpiCtx e = make_epi(p, bz);
   constexpr int ESZ = OUTCLS == OUT8 ? 1 : (OUTCLS == OUT32 ? 4 : 2);
   char* Cz = (char*)p.C + (int64_t)bz * p.sCb * ESZ;
   const int nch_mine = (NCH - kpart + KS - 1) / KS;  // chunks kpart, kpart + KS, ...
@@ -1670,7 +1674,7 @@ static int pick_config(const GemmParams& p) {
   if (p.M <= 16) {
     // one GEMM over a long K: stream the weights as whole row pieces; short K or batched (the
     // decode attention BMMs): MFMA-layout loads, two slabs per wave while enough waves remain
-    if (p.batch == 1 && p.K >= 1024) return CFG_ROWS4_16;
+    if (p.batch <= 4 && p.K >= 1024) return CFG_ROWS4_16;
     return (p.N + 31) / 32 >= 160 ? CFG_SKINNY_16_G2 : CFG_SKINNY_16;
   }
   if (p.M <= 64) return CFG_SKINNY_16 + (p.M > 16) + (p.M > 32);
@@ -1833,6 +1837,27 @@ int ti_bmm_i8_config(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk, con
   p.alpha = alpha; p.beta = beta;
   p.epilogue = epilogue; p.out_dtype = out_dtype; p.round_mode = round_mode;
   p.tiles_m = p.tiles_n = 0; p.group_m = 1; p.ksplit = 1;
+  p.bias_bs = 0; p.scale_bs = 0;
+  return ti::run(p, config, (hipStream_t)stream);
+}
+
+int ti_bmm_i8_grouped(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk, const int8_t* B, int64_t sBb,
+                      int64_t sBn, int64_t sBk, void* C, int64_t sCb, int64_t sCm, int64_t sCn, int batch, int M,
+                      int N, int K, const void* bias, int bias_kind, int64_t bias_batch_stride, const float* alpha,
+                      const float* beta, int64_t scale_batch_stride, int epilogue, int out_dtype, int round_mode,
+                      int config, void* stream) {
+  if (bias_batch_stride < 0 || scale_batch_stride < 0) return ti::fail(TI_E_STRIDE, "negative batch stride of bias or scales");
+  ti::GemmParams p;
+  p.A = A; p.B = B; p.C = C;
+  p.sAb = sAb; p.sAm = sAm; p.sAk = sAk;
+  p.sBb = sBb; p.sBn = sBn; p.sBk = sBk;
+  p.sCb = sCb; p.sCm = sCm; p.sCn = sCn;
+  p.batch = batch; p.M = M; p.N = N; p.K = K;
+  p.bias = bias; p.bias_kind = bias_kind;
+  p.alpha = alpha; p.beta = beta;
+  p.epilogue = epilogue; p.out_dtype = out_dtype; p.round_mode = round_mode;
+  p.tiles_m = p.tiles_n = 0; p.group_m = 1; p.ksplit = 1;
+  p.bias_bs = bias_batch_stride; p.scale_bs = scale_batch_stride;
   return ti::run(p, config, (hipStream_t)stream);
 }
 

@@ -6,9 +6,11 @@ import torch
 from .. import _lib as L
 
 
-def _launch(a, sa, b, sb, c, sc, B, M, N, K, *, epilogue, bias, alpha, beta, round_mode, config):
+def _launch(a, sa, b, sb, c, sc, B, M, N, K, *, epilogue, bias, alpha, beta, round_mode, config, grouped=False):
     """One ti_bmm_i8_config call: a/b/c are tensors (for pointers, dtype, device), sa/sb/sc the
-    (batch, row, column) element strides of the logical [B,M,K] / [B,N,K] / [B,M,N] views."""
+    (batch, row, column) element strides of the logical [B,M,K] / [B,N,K] / [B,M,N] views.
+    grouped: the batches are B projections with their own bias rows ([B*N] elements) and their
+    own scales (alpha / beta are fp32 device tensors of B elements): ti_bmm_i8_grouped."""
     L.require_cuda(a, b, c, bias)
     assert a.dtype == torch.int8 and b.dtype == torch.int8, "operands must be int8"
     dev = a.device
@@ -17,11 +19,24 @@ def _launch(a, sa, b, sb, c, sc, B, M, N, K, *, epilogue, bias, alpha, beta, rou
     bias_ptr = 0
     if bias is not None:
         assert bias.device == dev
-        assert bias.numel() == N, "bias must have one element per output column"
+        assert bias.numel() == (B * N if grouped else N), "bias must have one element per output column"
         if not bias.is_contiguous():
             bias = bias.contiguous()
         bias_kind = L.TORCH_TO_BIAS[bias.dtype]
         bias_ptr = bias.data_ptr()
+    if grouped:
+        for t in (alpha, beta):
+            assert t is None or (t.dtype == torch.float32 and t.device == dev and t.numel() == B and t.is_contiguous()), \
+                "grouped scales must be fp32 device tensors with one element per projection"
+        with L.on_device(dev):
+            rc = L.lib().ti_bmm_i8_grouped(
+                a.data_ptr(), sa[0], sa[1], sa[2], b.data_ptr(), sb[0], sb[1], sb[2], c.data_ptr(), sc[0], sc[1], sc[2],
+                B, M, N, K, bias_ptr, bias_kind, N, 0 if alpha is None else alpha.data_ptr(),
+                0 if beta is None else beta.data_ptr(), 1,
+                int(epilogue), L.TORCH_TO_DT[c.dtype], int(round_mode), int(config), L.current_stream(dev))
+        if rc != 0:
+            L.check(rc, "ti_bmm_i8_grouped")
+        return
     alpha_ptr = 0 if alpha is None else L.scale_tensor(alpha, dev).data_ptr()
     beta_ptr = 0 if beta is None else L.scale_tensor(beta, dev).data_ptr()
     with L.on_device(dev):
@@ -83,3 +98,29 @@ def bmm(a, b, *, b_is_kn, epilogue, out_dtype, alpha=None, out=None, round_mode=
         c = out
     launch_bmm(a, b, c, epilogue=epilogue, alpha=alpha, round_mode=round_mode, config=config)
     return c.view(*tmp_shape, N)
+
+
+def linear_group(a, w, groups, *, epilogue, out_dtype, bias=None, alpha=None, beta=None, out=None,
+                 round_mode=L.ROUND_RNE_CLAMP, config=-1):
+    """`groups` linears that share the input, as one launch: w is their [N,K] weights stacked to
+    [groups*N, K], bias [groups*N], alpha / beta fp32 device tensors [groups].  Returns
+    [*, groups*N]: projection g is columns g*N .. g*N+N.  Same arithmetic per projection as
+    `linear` (reference: kernels/linear.py:257-288 launched once per projection)."""
+    tmp_shape = a.shape[:-1]
+    assert len(w.shape) == 2 and w.shape[0] % groups == 0
+    assert a.shape[-1] == w.shape[1], "Incompatible dimensions"
+    GN, K = w.shape
+    N = GN // groups
+    M = 1
+    for d in tmp_shape:
+        M *= d
+    a = a.view(M, K)
+    if out is None:
+        c = torch.empty((M, GN), device=a.device, dtype=out_dtype)
+    else:
+        assert out.dtype == out_dtype and out.numel() == M * GN, "out has the wrong dtype or size"
+        c = out.view(M, GN)
+    _launch(a, (0, a.stride(0), a.stride(1)), w, (N * w.stride(0), w.stride(0), w.stride(1)),
+            c, (N * c.stride(1), c.stride(0), c.stride(1)), groups, M, N, K, epilogue=epilogue, bias=bias,
+            alpha=alpha, beta=beta, round_mode=round_mode, config=config, grouped=True)
+    return c.view(*tmp_shape, GN)

@@ -11,6 +11,7 @@ import torch
 
 from .. import _lib as L
 from ._gemm import linear as _linear
+from ._gemm import linear_group as _linear_group
 
 
 def linear_a8_w8_ofp32(a, b, scale, out=None, dtype=torch.float, *, _config=-1):
@@ -22,6 +23,17 @@ def linear_a8_w8_b8_o8(a, b, bias, scale_a, scale_b, out=None, *, _round_mode=L.
     """q8(scale_a * acc + scale_b * bias_i8) (reference: kernels/linear.py:256-288)."""
     return _linear(a, b, epilogue=L.EPI_SCALE_I8, out_dtype=torch.int8, bias=bias, alpha=scale_a, beta=scale_b,
                    out=out, round_mode=_round_mode, config=_config)
+
+
+def linear_group_a8_w8_b8_o8(a, b, bias, scale_a, scale_b, groups, out=None, *, _config=-1):
+    """`groups` linear_a8_w8_b8_o8 projections of one input as a single launch (the q/k/v
+    projections of an attention block: three W8A8B8O8Linear, nn/linear.py:18-67, which the
+    reference launches one after the other).  b: the [N,K] weights stacked to [groups*N, K];
+    bias int8 [groups*N]; scale_a, scale_b: fp32 device tensors [groups].  Returns
+    [..., groups*N] int8, projection g in columns g*N .. g*N+N, each element exactly what
+    linear_a8_w8_b8_o8 gives for that projection."""
+    return _linear_group(a, b, groups, epilogue=L.EPI_SCALE_I8, out_dtype=torch.int8, bias=bias, alpha=scale_a,
+                         beta=scale_b, out=out, config=_config)
 
 
 def linear_relu_a8_w8_b8_o8(a, b, bias, scale_a, scale_b, out=None, *, _round_mode=L.ROUND_RNE_CLAMP, _config=-1):

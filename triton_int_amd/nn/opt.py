@@ -7,7 +7,7 @@ end-to-end tests: every heavy step is one of the package's HIP kernels, torch on
 
     hidden fp32 [B,S,H]
       LayerNormQ -> int8                                    (layer_norm_fwd_fused_single_pass_q)
-      q,k,v = W8A8B8O8Linear -> int8                        (linear_a8_w8_b8_o8)
+      q,k,v = 3 x W8A8B8O8Linear -> int8, one launch        (linear_group_a8_w8_b8_o8)
       scores = BMM_S8T_S8N_S8T(q, k) -> int8                (bmm_s8t_s8n_s8t)
       probs  = softmax_q(scores, causal) -> int8 [0,127]    (ti_softmax_q)
       ctx    = BMM_S8T_S8N_S8T(probs, v^T) -> int8, written head-merged through output strides
@@ -22,6 +22,7 @@ import torch
 
 from ..kernels.bmm import bmm_s8t_s8n_s8t
 from ..kernels.fused import softmax_q, transpose_i8
+from ..kernels.linear import linear_group_a8_w8_b8_o8
 from .fused import DQ_Add_LayerNorm_Q, LayerNormQ, W8A8BFP32OFP32_GeLu_Q
 from .linear import W8A8B8O8Linear, W8A8B32O32LinearWithoutScaling, W8A8BFP32OFP32Linear
 
@@ -71,6 +72,25 @@ class W8A8OPTDecoderLayer(torch.nn.Module):
             ln.bias = (torch.randn(self.hidden, generator=g) * 0.1).div(0.05).to(ln.bias.device)
         return self
 
+    def _qkv_pack(self):
+        """The three projections' weights, biases and scales stacked for the grouped launch.  Built
+        on first use and whenever one of the modules' tensors was replaced or moved; the modules'
+        weight / bias are then re-pointed at slices of the pack, so the weights exist once."""
+        mods = (self.q_proj, self.k_proj, self.v_proj)
+        key = tuple((m.weight.data_ptr(), m.bias.data_ptr(), m.a.data_ptr(), m.b.data_ptr()) for m in mods)
+        if getattr(self, "_qkv_key", None) != key:
+            H = self.hidden
+            w = torch.cat([m.weight for m in mods], dim=0).contiguous()
+            bias = torch.cat([m.bias for m in mods], dim=0).contiguous()
+            a = torch.stack([m.a.reshape(()) for m in mods]).to(torch.float32).contiguous()
+            b = torch.stack([m.b.reshape(()) for m in mods]).to(torch.float32).contiguous()
+            for i, m in enumerate(mods):
+                m.weight, m.bias = w[i * H:(i + 1) * H], bias[i * H:(i + 1) * H]
+                m.a, m.b = a[i], b[i]
+            self._qkv = (w, bias, a, b)
+            self._qkv_key = tuple((m.weight.data_ptr(), m.bias.data_ptr(), m.a.data_ptr(), m.b.data_ptr()) for m in mods)
+        return self._qkv
+
     def _heads(self, t, B, S):
         # [B,S,H] int8 -> [B*heads, S, D].  One batch: a strided view (the BMM takes row and batch
         # strides, each head's rows stay K-contiguous).  Several batches: a copy.
@@ -79,16 +99,23 @@ class W8A8OPTDecoderLayer(torch.nn.Module):
         return t.view(B, S, self.heads, self.head_dim).transpose(1, 2).reshape(B * self.heads, S, self.head_dim)
 
     @torch.no_grad()
-    def forward(self, hidden, kv_cache=None, _trace=None):
+    def forward(self, hidden, kv_cache=None, _trace=None, _mark=None):
         """hidden fp32 [B,S,H].  kv_cache = (K int8 [B*heads, T, D], V^T int8 [B*heads, D, T]) holds the
         T-S earlier positions in its first T-S slots; the S new positions are written into the last S
         slots before attention (decode / chunked prefill).  Returns fp32 [B,S,H].  A dict passed as
-        `_trace` receives every intermediate tensor (for stage-by-stage parity tests)."""
+        `_trace` receives every intermediate tensor (for stage-by-stage parity tests); a callable
+        passed as `_mark` is called with a stage name after that stage's launches (for timing the
+        stages in sequence with stream events)."""
+        mark = _mark if _mark is not None else (lambda name: None)
         B, S, H = hidden.shape
         h8 = self.ln1(hidden)
-        q = self._heads(self.q_proj(h8), B, S)
-        k_new = self._heads(self.k_proj(h8), B, S)
-        v = self.v_proj(h8)                                                        # [B,S,H] int8
+        mark("ln1_layernorm_q")
+        w3, b3, a3, s3 = self._qkv_pack()
+        qkv = linear_group_a8_w8_b8_o8(h8, w3, b3, a3, s3, 3)                       # [B,S,3H] int8
+        q = self._heads(qkv[..., :H], B, S)
+        k_new = self._heads(qkv[..., H:2 * H], B, S)
+        v = qkv[..., 2 * H:]                                                       # [B,S,H] int8, row pitch 3H
+        mark("qkv_3x_linear_o8")
         if kv_cache is None:
             k_all = k_new
             vt_all = torch.empty((B * self.heads, self.head_dim, S), dtype=torch.int8, device=hidden.device)
@@ -100,9 +127,12 @@ class W8A8OPTDecoderLayer(torch.nn.Module):
         # V^T of every head of a batch in one transpose: [S, heads*D] -> the last S columns of [heads*D, T]
         for b in range(B):
             transpose_i8(v[b], out=vt_all[b * self.heads:(b + 1) * self.heads].view(H, T)[:, T - S:])
+        mark("kv_append_v_transpose")
         T = k_all.shape[1]
         scores = bmm_s8t_s8n_s8t(q, k_all, self.qk_alpha)                           # [B*heads, S, T] int8
+        mark("qk_bmm_o8")
         probs = softmax_q(scores, self.score_scale, causal_q_len=S if self.causal else 0)
+        mark("softmax_q")
         # P.V with the head merge folded into the output strides: head h of batch b writes columns
         # h*D .. h*D+D of row (b, s) of a [B,S,H] tensor
         ctx = torch.empty((B, S, H), dtype=torch.int8, device=hidden.device)
@@ -110,11 +140,17 @@ class W8A8OPTDecoderLayer(torch.nn.Module):
             out_view = ctx[b].view(S, self.heads, self.head_dim).transpose(0, 1)   # [heads, S, D] strided
             bmm_s8t_s8n_s8t(probs[b * self.heads:(b + 1) * self.heads], vt_all[b * self.heads:(b + 1) * self.heads],
                             self.pv_alpha, out=out_view)
+        mark("pv_bmm_o8")
         acc = self.out_proj(ctx)                                                    # int32 [B,S,H]
+        mark("out_proj_linear_o32")
         resid, h8b = self.ln2(hidden, acc)
+        mark("ln2_dq_add_layernorm_q")
         f8 = self.fc1(h8b)
+        mark("fc1_linear_gelu_q")
         y = self.fc2(f8)
+        mark("fc2_linear_f32")
         out = y + resid
+        mark("residual_add")
         if _trace is not None:
             _trace.update(h8=h8, q=q, k_all=k_all, vt_all=vt_all, scores=scores, probs=probs, ctx=ctx, acc=acc,
                           resid=resid, h8b=h8b, f8=f8, fc2=y, out=out)
