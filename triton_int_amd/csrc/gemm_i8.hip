@@ -543,6 +543,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
 // WTN / 16 is a power of two (the swizzle below needs that), none otherwise (direct stores)
 constexpr int epi_strip_bytes(int wtn) { return ((wtn / 16) & (wtn / 16 - 1)) == 0 ? 32 * wtn : 0; }
 
+// 4-byte outputs: every store instruction writes two whole 128-byte lines, which go out non-temporal
+// (measured on the P.V shape with fp32 output: 192 -> 162 us)
+#ifndef TI_STREAM_STORE32_AUX
+#define TI_STREAM_STORE32_AUX 2
+#endif
 template <int TM, int TN, int OUTCLS>
 __device__ __forceinline__ void stream_epilogue(const GemmParams& p, const EpiCtx& e, v16i (&acc)[TM][TN], int bz,
                                                 int mw, int nw, char* strip, int lane) {
@@ -657,13 +662,13 @@ __device__ __forceinline__ void stream_epilogue(const GemmParams& p, const EpiCt
             const int off = (n_ok && m < p.M) ? (m * ldc + n) * ESZ : OOB;
             const int a = acc[i][j][r];
             if constexpr (KIND == 0) {
-              __builtin_amdgcn_raw_buffer_store_b32((unsigned)a + (unsigned)bias_i32, rC, off, 0, 0);
+              __builtin_amdgcn_raw_buffer_store_b32((unsigned)a + (unsigned)bias_i32, rC, off, 0, TI_STREAM_STORE32_AUX);
             } else {
               float v = (float)a * e.alpha;
               const float vb = col + v;
               v = has_bias ? vb : v;
-              if constexpr (KIND == 1) __builtin_amdgcn_raw_buffer_store_b32((unsigned)q32(v, e.round_mode), rC, off, 0, 0);
-              else if constexpr (KIND == 2) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rC, off, 0, 0);
+              if constexpr (KIND == 1) __builtin_amdgcn_raw_buffer_store_b32((unsigned)q32(v, e.round_mode), rC, off, 0, TI_STREAM_STORE32_AUX);
+              else if constexpr (KIND == 2) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rC, off, 0, TI_STREAM_STORE32_AUX);
               else if constexpr (KIND == 3) __builtin_amdgcn_raw_buffer_store_b16(f32_to_f16_bits(v), rC, off, 0, 0);
               else __builtin_amdgcn_raw_buffer_store_b16(f32_to_bf16_bits(v), rC, off, 0, 0);
             }
