@@ -1784,7 +1784,9 @@ static int run(GemmParams p, int config, hipStream_t stream) {
     // every wave of a workgroup gets the same number of units (they meet at a barrier per chunk
     // of K), and the workgroups fit the chip in one round
     const int slots = R4_NW / p.ksplit;
-    const int per = slots * ((units + slots * 256 - 1) / (slots * 256));
+    // fewer units than wave slots on the chip: spread them over all 256 CUs (some waves of a
+    // workgroup then have no unit; they only join the barriers)
+    const int per = units < slots * 256 ? (units + 255) / 256 : slots * ((units + slots * 256 - 1) / (slots * 256));
     const int blocks = (units + per - 1) / per;
     g_last_config = config;
     k.fn[out_class(p.out_dtype)]<<<dim3((unsigned)blocks, (unsigned)p.batch), dim3(k.threads), 0, stream>>>(p);
