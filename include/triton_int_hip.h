@@ -221,6 +221,29 @@ int ti_softmax_q(const int8_t* x, int64_t x_row_stride, float scale,
 int ti_transpose_i8(const int8_t* src, int64_t src_row_stride, int8_t* dst, int64_t dst_row_stride,
                     int rows, int cols, void* stream);
 
+/*
+ * One attention block without the score round trip through memory:
+ *     scores = q8(qk_alpha * (q . k^T))                    (bmm_s8t_s8n_s8t, kernels/bmm.py:576-612)
+ *     probs  = round_half_even(127 * softmax(scores * score_scale)), causal mask as ti_softmax_q
+ *     out    = q8(pv_alpha * (probs . v))                  (bmm_s8t_s8n_s8t again, b = V^T)
+ * q [batch, S, D], k [batch, T, D], vt [batch, D, T] (V^T, as the P.V BMM takes it), out
+ * [batch, S, D]; int8, unit stride along the last dimension, batch and row strides in elements
+ * (all multiples of 16, like the pointers); D = 128; T a multiple of 16; 0 < score_scale <= 0.32.
+ * The scalars are host floats.  The int8 scores are bit-identical to the BMM's; a probability can
+ * differ from ti_softmax_q's by one step where 127 * e / sum lies within fp32 rounding of a half
+ * (the row's exponentials are summed in a different order).  All columns of a row that share an
+ * int8 score flip together, so such a row (about 1 in 10^5 at 2048 keys) can differ from the
+ * three-launch result in several output values by a few steps; every other row is identical.
+ * The reference has no fused form (its modules stop at the BMMs, nn/bmm.py:10-74); the
+ * three-launch chain remains available and is what this is tested against.
+ */
+int ti_attention_i8(const int8_t* q, int64_t q_batch_stride, int64_t q_row_stride,
+                    const int8_t* k, int64_t k_batch_stride, int64_t k_row_stride,
+                    const int8_t* vt, int64_t vt_batch_stride, int64_t vt_row_stride,
+                    int8_t* out, int64_t out_batch_stride, int64_t out_row_stride,
+                    int batch, int S, int T, int D,
+                    float qk_alpha, float score_scale, float pv_alpha, int causal_q_len, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

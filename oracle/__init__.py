@@ -218,3 +218,13 @@ def softmax_q(x_i8, scale, causal_q_len=0):
     rc = lib().ti_oracle_softmax_q(_p(x2), i64(cols), ctypes.c_float(scale), _p(y), i64(cols), rows, cols, int(causal_q_len))
     assert rc == 0
     return y.reshape(x_i8.shape)
+
+
+def attention_i8(q, k, vt, qk_alpha, score_scale, pv_alpha, causal_q_len=0, return_all=False):
+    """The three steps an attention block chains (reference: nn/bmm.py:10-29 BMM_S8T_S8N_S8T for
+    Q.K^T, the caller's softmax, nn/bmm.py:10-29 again for P.V), restated as that chain:
+    int8 scores, int8 probabilities, int8 context.  q [BH,S,D], k [BH,T,D], vt [BH,D,T]."""
+    scores = bmm_s8t_s8n_s8t(q, k, np.float32(qk_alpha))
+    probs = softmax_q(scores, score_scale, causal_q_len=causal_q_len)
+    ctx = bmm_s8t_s8n_s8t(probs, vt, np.float32(pv_alpha))
+    return (scores, probs, ctx) if return_all else ctx

@@ -87,9 +87,26 @@ def test_decoder_layer_opt13b_shapes_run():
     layer = W8A8OPTDecoderLayer().randomize(seed=1).to(DEV)
     g = torch.Generator(device="cpu").manual_seed(2)
     hidden = torch.randn((1, 2048, 5120), generator=g)
+    # one-kernel attention (the default at this size) against the three-launch chain
+    trf = {}
+    out_fused = layer(hidden.to(DEV), _trace=trf)
+    assert trf["scores"] is None and trf["probs"] is None
+    layer.fused_attention = False
     tr = {}
     out = layer(hidden.to(DEV), _trace=tr)
     assert out.shape == (1, 2048, 5120) and torch.isfinite(out).all()
+    # The two paths sum a row's exponentials in different orders.  A probability whose exact value
+    # sits within fp32 rounding of k + 0.5 can come out one step apart, and every column of that
+    # row with the same int8 score flips with it, so a rare row (measured: 1 of 81 920 here) can
+    # differ in many context values; all other rows are identical.
+    diff = (trf["ctx"].int() - tr["ctx"].int()).abs()[0].view(2048, 40, 128)
+    bad_rows = int((diff.amax(dim=-1) > 0).sum())
+    print(f"fused vs chained attention context: {bad_rows} of {2048 * 40} rows differ, max diff {int(diff.max())}")
+    assert bad_rows <= 8 and int(diff.max()) <= 16
+    assert torch.equal(trf["q"], tr["q"]) and torch.equal(trf["vt_all"], tr["vt_all"])
+    # everything after attention works row by row: the layer outputs differ in those token rows only
+    bad_tokens = diff.amax(dim=(1, 2)) > 0
+    assert torch.equal(out_fused[0][~bad_tokens], out[0][~bad_tokens])
     rows = [0, 777, 2047]
     h8 = cpu(tr["h8"])[0]
     q = O.linear_a8_w8_b8_o8(h8[rows], cpu(layer.q_proj.weight), cpu(layer.q_proj.bias), np.float32(float(layer.q_proj.a)), np.float32(float(layer.q_proj.b)))

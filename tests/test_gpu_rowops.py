@@ -194,3 +194,56 @@ def test_transpose_i8(rows, cols):
     fused.transpose_i8(gpu(x), out=gc[:, T - rows:])
     want = cache.copy(); want[:, T - rows:] = x.T
     assert np.array_equal(cpu(gc), want)
+
+
+@pytest.mark.parametrize("BH,S,T,q_len", [(3, 128, 128, 128), (2, 200, 336, 0), (2, 48, 272, 48), (1, 16, 2048, 16),
+                                           (2, 300, 300 + 4, 0), (4, 256, 256, 64), (1, 1, 16, 0)])
+def test_attention_i8_against_the_three_kernel_chain(BH, S, T, q_len):
+    """Fused Q.K^T -> softmax -> P.V.  The checker is the oracle's chain of the three steps.  The
+    int8 scores inside the kernel are the BMM's bit for bit, so differences can only come from
+    probabilities that sit on a rounding boundary (allowed: one step, rarely) and what they do to a
+    context value (one step)."""
+    fused = _fused()
+    T = (T + 15) // 16 * 16
+    g = rng(BH * 1000 + S + T)
+    D = 128
+    q = g.integers(-127, 128, size=(BH, S, D), dtype=np.int8)
+    k = g.integers(-127, 128, size=(BH, T, D), dtype=np.int8)
+    vt = g.integers(-127, 128, size=(BH, D, T), dtype=np.int8)
+    seen_nontrivial = False
+    for qk_alpha, score_scale, pv_alpha in ((1e-3, 0.05, 1.0 / 127.0), (4e-3, 0.02, 0.03)):
+        want = O.attention_i8(q, k, vt, qk_alpha, score_scale, pv_alpha, causal_q_len=q_len)
+        got = cpu(fused.attention_i8(gpu(q), gpu(k), gpu(vt), qk_alpha, score_scale, pv_alpha, causal_q_len=q_len))
+        mx, rate = mismatch_report(got, want)
+        print(f"attention_i8 BH {BH} S {S} T {T} q_len {q_len} alpha {qk_alpha}: max diff {mx}, mismatch rate {rate:.2e}")
+        bad_rows = int((np.abs(got.astype(int) - want.astype(int)).max(axis=-1) > 0).sum())
+        assert got.shape == (BH, S, D) and bad_rows <= max(1, BH * S // 1000), f"{bad_rows} rows differ (max {mx})"
+        seen_nontrivial = seen_nontrivial or np.unique(got).size > 8
+    assert seen_nontrivial or T >= 1024  # long rows of random scores spread the probabilities below 1/254
+
+
+def test_attention_i8_strided_views_and_errors():
+    fused = _fused()
+    g = rng(77)
+    S, heads, D, T = 160, 3, 128, 160
+    # the layer's layouts: q / k as head views of a [S, heads*D] projection, out head-merged
+    qflat = g.integers(-127, 128, size=(S, heads * D), dtype=np.int8)
+    kflat = g.integers(-127, 128, size=(T, heads * D), dtype=np.int8)
+    vt_wide = g.integers(-127, 128, size=(heads, D, T + 32), dtype=np.int8)
+    vt = vt_wide[:, :, :T]
+    gq = gpu(qflat).view(S, heads, D).transpose(0, 1)
+    gk = gpu(kflat).view(T, heads, D).transpose(0, 1)
+    gvt = gpu(vt_wide)[:, :, :T]  # row pitch T + 32
+    out = torch.zeros((S, heads * D), dtype=torch.int8, device=DEV)
+    fused.attention_i8(gq, gk, gvt, 1e-3, 0.05, 1.0 / 127.0, causal_q_len=S,
+                       out=out.view(S, heads, D).transpose(0, 1))
+    q3 = qflat.reshape(S, heads, D).transpose(1, 0, 2)
+    k3 = kflat.reshape(T, heads, D).transpose(1, 0, 2)
+    want = O.attention_i8(np.ascontiguousarray(q3), np.ascontiguousarray(k3), np.ascontiguousarray(vt), 1e-3, 0.05,
+                          1.0 / 127.0, causal_q_len=S)
+    mx, rate = mismatch_report(cpu(out).reshape(S, heads, D).transpose(1, 0, 2), want)
+    assert mx <= 1 and rate < 5e-3
+    with pytest.raises(AssertionError):  # head dimension other than 128
+        fused.attention_i8(gpu(q3[:, :, :64].copy()), gpu(k3[:, :, :64].copy()), gpu(vt[:, :64].copy()), 1e-3, 0.05, 0.01)
+    with pytest.raises(AssertionError):  # score scale too large for the fixed-bound exponent
+        fused.attention_i8(gq, gk, gvt, 1e-3, 0.5, 0.01)

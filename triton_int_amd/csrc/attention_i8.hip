@@ -1,0 +1,313 @@
+// attention_i8.hip — int8 attention for one block of query rows without the score round trip.
+//
+// The reference's callers chain three launches per attention block (nn/bmm.py:10-29 for Q.K^T,
+// a softmax in the caller, nn/bmm.py:10-29 / :54-74 for P.V):
+//     scores = q8(qk_alpha * (q . k))                      int8 [BH, S, T]   (kernels/bmm.py:576-612)
+//     probs  = rne(127 * softmax(scores * score_scale))    int8 [BH, S, T]   values 0..127
+//     ctx    = q8(pv_alpha * (probs . v))                  int8 [BH, S, D]   (kernels/bmm.py:576-612)
+// At 2048 x 2048 scores per head the two intermediates are 4 x 168 MB of HBM traffic for 40 heads.
+// This kernel computes the same three steps per 32 x 32 block of scores in registers: the int8
+// score quantisation, the probability quantisation and the context quantisation are the same
+// fp32 operations as in the three kernels; only the order in which a row's exponentials are
+// summed differs (and the exponent is taken against the fixed bound 127 instead of the row
+// maximum, which cancels in the quotient), so a probability can differ by one step when
+// 127 * e / sum falls within rounding error of a half; every column of that row with the same
+// int8 score then flips with it, and the row's context values can move by a few steps (measured:
+// 1 row of 81 920 at 2048 keys; all other rows bit-identical to the three-kernel chain).
+//
+// Two passes over the keys of a query block, as the probabilities need the whole row's sum before
+// they can be quantised: pass 1 computes scores and sums exponentials, pass 2 recomputes the
+// scores (K = 128 deep: cheap), forms the int8 probabilities in the MFMA operand layout straight
+// from the accumulator registers and feeds them to the P.V MFMAs.  The order of the keys inside
+// a 32-key block is a free choice (it is the reduction index of P.V): V^T is stored to LDS in
+// the order in which the score accumulators hold the keys, so P never moves between lanes.
+//
+// Workgroup = 4 waves = 128 query rows of one head; a wave owns 32 rows.  K and V^T are staged
+// through LDS in tiles of 64 keys, double-buffered, one barrier per tile.  Causal masking skips
+// whole key tiles beyond a wave's last visible key and masks inside the tiles on the diagonal.
+#include <type_traits>
+
+#include "ti_common.h"
+
+namespace ti {
+
+constexpr int AT_D = 128;                // head dimension this kernel is written for
+constexpr int AT_ROWS = 128;             // query rows per workgroup
+constexpr int AT_KT = 64;                // keys per LDS tile
+constexpr int AT_KP = AT_D + 16;         // K tile row pitch (bytes): 16-byte reads of 16 rows hit 64 different banks
+constexpr int AT_VP = AT_KT + 16;        // V^T tile row pitch
+constexpr int AT_KBYTES = AT_KT * AT_KP;
+constexpr int AT_VBYTES = AT_D * AT_VP;
+
+struct AttnParams {
+  const int8_t* q; const int8_t* k; const int8_t* vt; int8_t* out;
+  int64_t sQb, sQm, sKb, sKn, sVb, sVd, sOb, sOm;
+  int S, T, causal_q_len, nblk, batch;
+  float qk_alpha, s2, pv_alpha;  // s2 = score_scale * log2(e)
+};
+
+__device__ __forceinline__ int attn_limit(const AttnParams& p, int row) {
+  return p.causal_q_len > 0 ? min(p.T, (row % p.causal_q_len) + (p.T - p.causal_q_len) + 1) : p.T;
+}
+
+__global__ __launch_bounds__(256, 2) void attention_i8_kernel(AttnParams p) {
+  __shared__ __attribute__((aligned(16))) char lds[2 * (AT_KBYTES + AT_VBYTES)];
+  __shared__ int wg_lim[4];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lrow = lane & 31, lhi = lane >> 5;
+  // Work item = (head, block of 128 query rows).  Under a causal mask a later row block sees more
+  // keys, and every workgroup of a launch of this size is resident at once, workgroup i on the same
+  // CU as i + 256 and i + 512 (measured placement).  The items are therefore taken in order of
+  // decreasing work and dealt to the workgroup indices in a snake: 0..255 forward, 256..511
+  // backward, ..., which gives every CU about the same total.
+  const int n_items = p.nblk * p.batch;
+  const int pass = (int)blockIdx.x >> 8, c = (int)blockIdx.x & 255;
+  const int cnt = min(256, n_items - pass * 256);
+  const int pos = pass * 256 + ((pass & 1) ? cnt - 1 - c : c);
+  const int bh = pos % p.batch;
+  const int m0 = (p.nblk - 1 - pos / p.batch) * AT_ROWS + wave * 32;
+  const int8_t* qb = p.q + (int64_t)bh * p.sQb;
+  const int8_t* kb_ = p.k + (int64_t)bh * p.sKb;
+  const int8_t* vb = p.vt + (int64_t)bh * p.sVb;
+
+  // ---- per-lane row, visible-key limit; wave and workgroup bounds
+  const int row = m0 + lrow;
+  const int rowc = min(row, p.S - 1);                       // rows past S repeat the last row, never stored
+  const int lim_lane = attn_limit(p, min(max(rowc, 0), p.S - 1));
+  int lim_hi = lim_lane, lim_lo = lim_lane;
+#pragma unroll
+  for (int off = 16; off > 0; off >>= 1) {
+    lim_hi = max(lim_hi, __shfl_xor(lim_hi, off, 64));
+    lim_lo = min(lim_lo, __shfl_xor(lim_lo, off, 64));
+  }
+  lim_hi = __builtin_amdgcn_readfirstlane(lim_hi);
+  lim_lo = __builtin_amdgcn_readfirstlane(lim_lo);
+  const bool wave_live = m0 < p.S;                          // a wave wholly past S computes nothing
+  if (lane == 0) wg_lim[wave] = wave_live ? lim_hi : 0;
+  __syncthreads();
+  const int wg_hi = max(max(wg_lim[0], wg_lim[1]), max(wg_lim[2], wg_lim[3]));
+  const int ntiles = __builtin_amdgcn_readfirstlane((wg_hi + AT_KT - 1) / AT_KT);
+
+  // ---- this wave's Q fragments (32 rows x 128 d): lane (row, half) holds 16 bytes per 32-deep step
+  v4i qf[4];
+#pragma unroll
+  for (int ds = 0; ds < 4; ++ds)
+    qf[ds] = *(const v4i*)(qb + (int64_t)rowc * p.sQm + ds * 32 + lhi * 16);
+
+  // ---- tile staging: thread t copies two 16-byte chunks of the K tile and two of the V^T tile
+  v4i kreg[2], vreg[2];
+  auto fetch = [&](int t, bool with_v) {
+    const int key0 = t * AT_KT;
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const int q_ = c * 256 + tid;          // chunk index: 64 keys x 8 chunks
+      const int kr = q_ >> 3, kc = q_ & 7;
+      const bool in = key0 + kr < p.T;
+      kreg[c] = in ? *(const v4i*)(kb_ + (int64_t)(key0 + kr) * p.sKn + kc * 16) : (v4i){0, 0, 0, 0};
+    }
+    if (with_v) {
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        const int q_ = c * 256 + tid;        // chunk index: 128 d x 4 chunks of 16 keys
+        const int vr = q_ >> 2, vc = q_ & 3;
+        const bool in = key0 + vc * 16 < p.T;  // T % 16 == 0: a chunk is wholly inside or outside
+        vreg[c] = in ? *(const v4i*)(vb + (int64_t)vr * p.sVd + key0 + vc * 16) : (v4i){0, 0, 0, 0};
+      }
+    }
+  };
+  auto stash = [&](int buf, bool with_v) {
+    char* kt = lds + buf * (AT_KBYTES + AT_VBYTES);
+    char* vt = kt + AT_KBYTES;
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const int q_ = c * 256 + tid;
+      *(v4i*)(kt + (q_ >> 3) * AT_KP + (q_ & 7) * 16) = kreg[c];
+    }
+    if (with_v) {
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        const int q_ = c * 256 + tid;
+        const int vr = q_ >> 2, vc = q_ & 3;
+        // keys 16*vc + 4*w .. +3 (dword w) of their 32-key block are held by the score
+        // accumulators of lane half (w & 1) as register group g = 2*(vc & 1) + (w >> 1):
+        // they go to byte 16*(w & 1) + 4*g of the block
+        char* dst = vt + vr * AT_VP + (vc >> 1) * 32;
+#pragma unroll
+        for (int w = 0; w < 4; ++w)
+          *(int*)(dst + 16 * (w & 1) + 4 * (2 * (vc & 1) + (w >> 1))) = vreg[c][w];
+      }
+    }
+  };
+
+  const float MAGIC = 12582912.0f;  // 1.5 * 2^23: adding it rounds to the nearest even integer
+  const float c127 = -(127.0f * p.s2);
+  // scores of one 32-key block -> exponentials e[r]; key of register r: 8*(r/4) + 4*lhi + r%4
+  auto score_exp_t = [&](const char* kt, int kblk, int key_base, float (&e)[16], auto mask_tag) {
+    constexpr bool MASK = decltype(mask_tag)::value;
+    v16i s;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] = 0;
+#pragma unroll
+    for (int ds = 0; ds < 4; ++ds) {
+      const v4i kf = *(const v4i*)(kt + (kblk * 32 + lrow) * AT_KP + ds * 32 + lhi * 16);
+      s = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qf[ds], s, 0, 0, 0);  // rows of the result = keys
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      float v = (float)s[r] * p.qk_alpha;
+      v = __builtin_amdgcn_fmed3f(v, -128.0f, 127.0f);
+      const float x = __builtin_rintf(v);  // the int8 score, as a float (round half to even, like the BMM's)
+      e[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x, p.s2, c127));
+    }
+    if constexpr (MASK) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = key_base + 8 * (r >> 2) + 4 * lhi + (r & 3);
+        e[r] = key < lim_lane ? e[r] : 0.0f;
+      }
+    }
+  };
+  // Off the diagonal no row's limit falls inside or before the block and the selects above must
+  // cost nothing: two instantiations behind a wave-uniform branch (the MFMAs inside keep the
+  // compiler from folding them back into one block of selects).
+  auto score_exp = [&](const char* kt, int kblk, int key_base, float (&e)[16]) {
+    if (key_base + 32 > lim_lo) score_exp_t(kt, kblk, key_base, e, std::true_type{});
+    else score_exp_t(kt, kblk, key_base, e, std::false_type{});
+  };
+
+  // ================= pass 1: row sums =================
+  float sum = 0.0f;
+  fetch(0, false);
+  stash(0, false);
+  __syncthreads();
+  for (int t = 0; t < ntiles; ++t) {
+    if (t + 1 < ntiles) fetch(t + 1, false);
+    const char* kt = lds + (t & 1) * (AT_KBYTES + AT_VBYTES);
+    if (wave_live) {
+#pragma unroll
+      for (int kblk = 0; kblk < 2; ++kblk) {
+        const int key_base = t * AT_KT + kblk * 32;
+        if (key_base < lim_hi) {
+          float e[16];
+          score_exp(kt, kblk, key_base, e);
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sum += e[r];
+        }
+      }
+    }
+    if (t + 1 < ntiles) stash((t + 1) & 1, false);
+    __syncthreads();
+  }
+  sum += __shfl_xor(sum, 32, 64);  // the two lane halves hold different keys of the same row
+  const float rinv = 127.0f / sum;
+
+  // ================= pass 2: probabilities and P.V =================
+  v16i o[4];
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[db][r] = 0;
+  fetch(0, true);
+  stash(0, true);
+  __syncthreads();
+  for (int t = 0; t < ntiles; ++t) {
+    if (t + 1 < ntiles) fetch(t + 1, true);
+    const char* kt = lds + (t & 1) * (AT_KBYTES + AT_VBYTES);
+    const char* vt = kt + AT_KBYTES;
+    if (wave_live) {
+#pragma unroll
+      for (int kblk = 0; kblk < 2; ++kblk) {
+        const int key_base = t * AT_KT + kblk * 32;
+        if (key_base < lim_hi) {
+          float e[16];
+          score_exp(kt, kblk, key_base, e);
+          v4i pf;  // 16 int8 probabilities of this lane's row, keys in accumulator order
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const unsigned b0 = __float_as_uint(__builtin_fmaf(e[4 * g + 0], rinv, MAGIC));
+            const unsigned b1 = __float_as_uint(__builtin_fmaf(e[4 * g + 1], rinv, MAGIC));
+            const unsigned b2 = __float_as_uint(__builtin_fmaf(e[4 * g + 2], rinv, MAGIC));
+            const unsigned b3 = __float_as_uint(__builtin_fmaf(e[4 * g + 3], rinv, MAGIC));
+            pf[g] = (int)(__builtin_amdgcn_perm(b1, b0, 0x0c0c0400u) | __builtin_amdgcn_perm(b3, b2, 0x04000c0cu));
+          }
+#pragma unroll
+          for (int db = 0; db < 4; ++db) {
+            const v4i vf = *(const v4i*)(vt + (db * 32 + lrow) * AT_VP + kblk * 32 + lhi * 16);
+            o[db] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf, pf, o[db], 0, 0, 0);  // rows of the result = d
+          }
+        }
+      }
+    }
+    if (t + 1 < ntiles) stash((t + 1) & 1, true);
+    __syncthreads();
+  }
+
+  // ---- context: o[db][r] is row lrow, d = 32*db + 8*(r/4) + 4*lhi + r%4 -> int8, 16 bytes per lane
+  if (!wave_live) return;
+  int8_t* ob = p.out + (int64_t)bh * p.sOb;
+#pragma unroll
+  for (int db = 0; db < 4; ++db) {
+    unsigned X[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      unsigned b[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        float v = (float)o[db][4 * g + t] * p.pv_alpha;
+        v = __builtin_amdgcn_fmed3f(v, -128.0f, 127.0f);
+        b[t] = __float_as_uint(v + MAGIC);
+      }
+      X[g] = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u) | __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);
+    }
+    // lanes l and l+32 hold alternate 4-byte groups of the row's 32 bytes: after the two swaps
+    // lane l has bytes 0..15 and lane l+32 bytes 16..31
+    const auto s02 = __builtin_amdgcn_permlane32_swap(X[0], X[2], false, false);
+    const auto s13 = __builtin_amdgcn_permlane32_swap(X[1], X[3], false, false);
+    v4u v;
+    v[0] = s02[0]; v[1] = s02[1]; v[2] = s13[0]; v[3] = s13[1];
+    if (row < p.S) *(v4u*)(ob + (int64_t)row * p.sOm + db * 32 + lhi * 16) = v;
+  }
+}
+
+}  // namespace ti
+
+extern "C" int ti_attention_i8(const int8_t* q, int64_t q_batch_stride, int64_t q_row_stride, const int8_t* k,
+                               int64_t k_batch_stride, int64_t k_row_stride, const int8_t* vt,
+                               int64_t vt_batch_stride, int64_t vt_row_stride, int8_t* out, int64_t out_batch_stride,
+                               int64_t out_row_stride, int batch, int S, int T, int D, float qk_alpha,
+                               float score_scale, float pv_alpha, int causal_q_len, void* stream) {
+  using namespace ti;
+  if (batch < 0 || S < 0 || T < 0 || causal_q_len < 0) return fail(TI_E_SHAPE, "negative size");
+  if (batch == 0 || S == 0) return TI_OK;
+  if (!q || !k || !vt || !out) return fail(TI_E_NULL, "q, k, vt and out are required");
+  if (D != AT_D) return fail(TI_E_SHAPE, "head dimension %d: this kernel is built for %d", D, AT_D);
+  if (T <= 0 || (T & 15)) return fail(TI_E_SHAPE, "T = %d must be a positive multiple of 16", T);
+  if (batch > 65535) return fail(TI_E_SHAPE, "batch %d > 65535", batch);
+  if (causal_q_len > T) return fail(TI_E_SHAPE, "causal_q_len %d > T %d", causal_q_len, T);
+  if (causal_q_len > 0 && S % causal_q_len) return fail(TI_E_SHAPE, "S %d not a multiple of causal_q_len %d", S, causal_q_len);
+  if (q_row_stride < D || k_row_stride < D || out_row_stride < D || vt_row_stride < T)
+    return fail(TI_E_STRIDE, "row strides must cover a row");
+  const uintptr_t align = (uintptr_t)q | (uintptr_t)k | (uintptr_t)vt | (uintptr_t)out | (uintptr_t)q_batch_stride |
+                          (uintptr_t)q_row_stride | (uintptr_t)k_batch_stride | (uintptr_t)k_row_stride |
+                          (uintptr_t)vt_batch_stride | (uintptr_t)vt_row_stride | (uintptr_t)out_batch_stride |
+                          (uintptr_t)out_row_stride;
+  if (align & 15) return fail(TI_E_STRIDE, "pointers and strides must be multiples of 16 bytes");
+  // exponentials are taken against the largest possible score (127): the smallest one must stay a
+  // normal fp32 number
+  const float s2 = score_scale * 1.44269504088896340736f;
+  if (!(score_scale > 0.0f) || s2 * 255.0f > 120.0f)
+    return fail(TI_E_COMBO, "score_scale %g outside (0, 0.32]: use the three-kernel path", (double)score_scale);
+  int rc = check_device();
+  if (rc != TI_OK) return rc;
+  AttnParams p;
+  p.q = q; p.k = k; p.vt = vt; p.out = out;
+  p.sQb = q_batch_stride; p.sQm = q_row_stride; p.sKb = k_batch_stride; p.sKn = k_row_stride;
+  p.sVb = vt_batch_stride; p.sVd = vt_row_stride; p.sOb = out_batch_stride; p.sOm = out_row_stride;
+  p.S = S; p.T = T; p.causal_q_len = causal_q_len;
+  p.qk_alpha = qk_alpha; p.s2 = s2; p.pv_alpha = pv_alpha;
+  p.nblk = (S + AT_ROWS - 1) / AT_ROWS;
+  p.batch = batch;
+  attention_i8_kernel<<<dim3((unsigned)(p.nblk * batch)), dim3(256), 0, (hipStream_t)stream>>>(p);
+  return launch_status("attention_i8_kernel");
+}

@@ -141,3 +141,29 @@ def transpose_i8(src, out=None):
                                      L.current_stream(src.device))
     L.check(rc, "ti_transpose_i8")
     return out
+
+
+def attention_i8(q, k, vt, qk_alpha, score_scale, pv_alpha, causal_q_len=0, out=None):
+    """bmm_s8t_s8n_s8t(q, k, qk_alpha) -> softmax_q(., score_scale, causal_q_len) ->
+    bmm_s8t_s8n_s8t(probs, vt, pv_alpha) as one kernel that keeps scores and probabilities in
+    registers (reference: the same three steps are separate launches, kernels/bmm.py:576-612 twice
+    plus the caller's softmax).  q [BH,S,128], k [BH,T,128], vt [BH,128,T] int8 with unit stride
+    along the last dimension; `out` may be any int8 [BH,S,128] view with unit last stride (e.g. the
+    head-merged [S, heads, 128] layout).  Scalars are python floats."""
+    L.require_cuda(q, k, vt, out)
+    assert q.dtype == torch.int8 and k.dtype == torch.int8 and vt.dtype == torch.int8, "operands must be int8"
+    assert q.dim() == 3 and k.dim() == 3 and vt.dim() == 3, "q, k, vt must be 3-D"
+    BH, S, D = q.shape
+    T = k.shape[1]
+    assert k.shape == (BH, T, D) and vt.shape == (BH, D, T), "Incompatible dimensions"
+    assert q.stride(2) == 1 and k.stride(2) == 1 and vt.stride(2) == 1, "unit stride along the last dimension"
+    if out is None:
+        out = torch.empty((BH, S, D), dtype=torch.int8, device=q.device)
+    assert out.dtype == torch.int8 and tuple(out.shape) == (BH, S, D) and out.stride(2) == 1
+    with L.on_device(q.device):
+        rc = L.lib().ti_attention_i8(L.ptr(q), q.stride(0), q.stride(1), L.ptr(k), k.stride(0), k.stride(1),
+                                     L.ptr(vt), vt.stride(0), vt.stride(1), L.ptr(out), out.stride(0), out.stride(1),
+                                     BH, S, T, D, float(qk_alpha), float(score_scale), float(pv_alpha),
+                                     int(causal_q_len), L.current_stream(q.device))
+    L.check(rc, "ti_attention_i8")
+    return out

@@ -11,6 +11,8 @@ end-to-end tests: every heavy step is one of the package's HIP kernels, torch on
       scores = BMM_S8T_S8N_S8T(q, k) -> int8                (bmm_s8t_s8n_s8t)
       probs  = softmax_q(scores, causal) -> int8 [0,127]    (ti_softmax_q)
       ctx    = BMM_S8T_S8N_S8T(probs, v^T) -> int8, written head-merged through output strides
+               (with `fused_attention`, the default for 128 or more query positions, these three run
+               as one kernel, ti_attention_i8, and scores / probabilities never reach memory)
       acc    = W8A8B32O32LinearWithoutScaling(ctx) -> int32 (linear_a8_w8_b32_o32)   out_proj
       resid, h8 = DQ_Add_LayerNorm_Q(hidden, acc)           (ti_dq_add_layernorm_q)
       f8     = W8A8BFP32OFP32_GeLu_Q(h8) -> int8            (GEMM + GELU-quant epilogue)   fc1
@@ -21,7 +23,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels.bmm import bmm_s8t_s8n_s8t
-from ..kernels.fused import softmax_q, transpose_i8
+from ..kernels.fused import attention_i8, softmax_q, transpose_i8
 from ..kernels.linear import linear_group_a8_w8_b8_o8
 from .fused import DQ_Add_LayerNorm_Q, LayerNormQ, W8A8BFP32OFP32_GeLu_Q
 from .linear import W8A8B8O8Linear, W8A8B32O32LinearWithoutScaling, W8A8BFP32OFP32Linear
@@ -45,6 +47,10 @@ class W8A8OPTDecoderLayer(torch.nn.Module):
         self.qk_alpha = 1e-3
         self.score_scale = 0.05
         self.pv_alpha = 1.0 / 127.0
+        # one-kernel attention for prefill-sized blocks of queries; the three-launch chain otherwise
+        # (a handful of query rows per head leaves that kernel too few workgroups)
+        self.fused_attention = True
+        self.fused_attention_min_queries = 128
 
     @torch.no_grad()
     def randomize(self, seed=0):
@@ -129,18 +135,29 @@ class W8A8OPTDecoderLayer(torch.nn.Module):
             transpose_i8(v[b], out=vt_all[b * self.heads:(b + 1) * self.heads].view(H, T)[:, T - S:])
         mark("kv_append_v_transpose")
         T = k_all.shape[1]
-        scores = bmm_s8t_s8n_s8t(q, k_all, self.qk_alpha)                           # [B*heads, S, T] int8
-        mark("qk_bmm_o8")
-        probs = softmax_q(scores, self.score_scale, causal_q_len=S if self.causal else 0)
-        mark("softmax_q")
-        # P.V with the head merge folded into the output strides: head h of batch b writes columns
-        # h*D .. h*D+D of row (b, s) of a [B,S,H] tensor
         ctx = torch.empty((B, S, H), dtype=torch.int8, device=hidden.device)
-        for b in range(B):
-            out_view = ctx[b].view(S, self.heads, self.head_dim).transpose(0, 1)   # [heads, S, D] strided
-            bmm_s8t_s8n_s8t(probs[b * self.heads:(b + 1) * self.heads], vt_all[b * self.heads:(b + 1) * self.heads],
-                            self.pv_alpha, out=out_view)
-        mark("pv_bmm_o8")
+        fused = (self.fused_attention and S >= self.fused_attention_min_queries and self.head_dim == 128
+                 and T % 16 == 0 and 0.0 < self.score_scale <= 0.32)
+        scores = probs = None
+        if fused:
+            for b in range(B):
+                hs = slice(b * self.heads, (b + 1) * self.heads)
+                attention_i8(q[hs], k_all[hs], vt_all[hs], self.qk_alpha, self.score_scale, self.pv_alpha,
+                             causal_q_len=S if self.causal else 0,
+                             out=ctx[b].view(S, self.heads, self.head_dim).transpose(0, 1))
+            mark("attention_i8_fused")
+        else:
+            scores = bmm_s8t_s8n_s8t(q, k_all, self.qk_alpha)                       # [B*heads, S, T] int8
+            mark("qk_bmm_o8")
+            probs = softmax_q(scores, self.score_scale, causal_q_len=S if self.causal else 0)
+            mark("softmax_q")
+            # P.V with the head merge folded into the output strides: head h of batch b writes columns
+            # h*D .. h*D+D of row (b, s) of a [B,S,H] tensor
+            for b in range(B):
+                out_view = ctx[b].view(S, self.heads, self.head_dim).transpose(0, 1)   # [heads, S, D] strided
+                bmm_s8t_s8n_s8t(probs[b * self.heads:(b + 1) * self.heads], vt_all[b * self.heads:(b + 1) * self.heads],
+                                self.pv_alpha, out=out_view)
+            mark("pv_bmm_o8")
         acc = self.out_proj(ctx)                                                    # int32 [B,S,H]
         mark("out_proj_linear_o32")
         resid, h8b = self.ln2(hidden, acc)
