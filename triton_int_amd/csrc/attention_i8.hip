@@ -142,38 +142,51 @@ __global__ __launch_bounds__(256, 2) void attention_i8_kernel(AttnParams p) {
 
   const float MAGIC = 12582912.0f;  // 1.5 * 2^23: adding it rounds to the nearest even integer
   const float c127 = -(127.0f * p.s2);
-  // scores of one 32-key block -> exponentials e[r]; key of register r: 8*(r/4) + 4*lhi + r%4
-  auto score_exp_t = [&](const char* kt, int kblk, int key_base, float (&e)[16], auto mask_tag) {
+  // Scores of one 64-key tile -> exponentials.  The tile's two 32-key blocks are two independent
+  // MFMA chains, interleaved, with all fragment reads issued first; e[b][r] belongs to key
+  // key0 + 32*b + 8*(r/4) + 4*lhi + r%4.  A block that lies wholly beyond the wave's last visible
+  // key is computed too and masked to zero (at most one per wave and pass).
+  auto score_exp_t = [&](const char* kt, int key0, float (&e)[2][16], auto mask_tag) {
     constexpr bool MASK = decltype(mask_tag)::value;
-    v16i s;
+    v4i kf[2][4];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) s[r] = 0;
+    for (int ds = 0; ds < 4; ++ds)
 #pragma unroll
-    for (int ds = 0; ds < 4; ++ds) {
-      const v4i kf = *(const v4i*)(kt + (kblk * 32 + lrow) * AT_KP + ds * 32 + lhi * 16);
-      s = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf, qf[ds], s, 0, 0, 0);  // rows of the result = keys
-    }
+      for (int b = 0; b < 2; ++b) kf[b][ds] = *(const v4i*)(kt + (b * 32 + lrow) * AT_KP + ds * 32 + lhi * 16);
+    v16i s[2];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      float v = (float)s[r] * p.qk_alpha;
-      v = __builtin_amdgcn_fmed3f(v, -128.0f, 127.0f);
-      const float x = __builtin_rintf(v);  // the int8 score, as a float (round half to even, like the BMM's)
-      e[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x, p.s2, c127));
-    }
-    if constexpr (MASK) {
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s[b][r] = 0;
+#pragma unroll
+    for (int ds = 0; ds < 4; ++ds)
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+        s[b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[b][ds], qf[ds], s[b], 0, 0, 0);  // rows of the result = keys
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int key = key_base + 8 * (r >> 2) + 4 * lhi + (r & 3);
-        e[r] = key < lim_lane ? e[r] : 0.0f;
+        float v = (float)s[b][r] * p.qk_alpha;
+        v = __builtin_amdgcn_fmed3f(v, -128.0f, 127.0f);
+        const float x = __builtin_rintf(v);  // the int8 score, as a float (round half to even, like the BMM's)
+        e[b][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x, p.s2, c127));
+      }
+      if constexpr (MASK) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = key0 + 32 * b + 8 * (r >> 2) + 4 * lhi + (r & 3);
+          e[b][r] = key < lim_lane ? e[b][r] : 0.0f;
+        }
       }
     }
   };
-  // Off the diagonal no row's limit falls inside or before the block and the selects above must
+  // Off the diagonal no row's limit falls inside or before the tile and the selects above must
   // cost nothing: two instantiations behind a wave-uniform branch (the MFMAs inside keep the
   // compiler from folding them back into one block of selects).
-  auto score_exp = [&](const char* kt, int kblk, int key_base, float (&e)[16]) {
-    if (key_base + 32 > lim_lo) score_exp_t(kt, kblk, key_base, e, std::true_type{});
-    else score_exp_t(kt, kblk, key_base, e, std::false_type{});
+  auto score_exp = [&](const char* kt, int key0, float (&e)[2][16]) {
+    if (key0 + AT_KT > lim_lo) score_exp_t(kt, key0, e, std::true_type{});
+    else score_exp_t(kt, key0, e, std::false_type{});
   };
 
   // ================= pass 1: row sums =================
@@ -184,17 +197,16 @@ __global__ __launch_bounds__(256, 2) void attention_i8_kernel(AttnParams p) {
   for (int t = 0; t < ntiles; ++t) {
     if (t + 1 < ntiles) fetch(t + 1, false);
     const char* kt = lds + (t & 1) * (AT_KBYTES + AT_VBYTES);
-    if (wave_live) {
+    if (wave_live && t * AT_KT < lim_hi) {
+      float e[2][16];
+      score_exp(kt, t * AT_KT, e);
+      float s0 = 0.0f, s1 = 0.0f;
 #pragma unroll
-      for (int kblk = 0; kblk < 2; ++kblk) {
-        const int key_base = t * AT_KT + kblk * 32;
-        if (key_base < lim_hi) {
-          float e[16];
-          score_exp(kt, kblk, key_base, e);
-#pragma unroll
-          for (int r = 0; r < 16; ++r) sum += e[r];
-        }
+      for (int r = 0; r < 16; ++r) {
+        s0 += e[0][r];
+        s1 += e[1][r];
       }
+      sum += s0 + s1;
     }
     if (t + 1 < ntiles) stash((t + 1) & 1, false);
     __syncthreads();
@@ -215,29 +227,30 @@ __global__ __launch_bounds__(256, 2) void attention_i8_kernel(AttnParams p) {
     if (t + 1 < ntiles) fetch(t + 1, true);
     const char* kt = lds + (t & 1) * (AT_KBYTES + AT_VBYTES);
     const char* vt = kt + AT_KBYTES;
-    if (wave_live) {
+    if (wave_live && t * AT_KT < lim_hi) {
+      float e[2][16];
+      score_exp(kt, t * AT_KT, e);
+      v4i vf[2][4];
 #pragma unroll
-      for (int kblk = 0; kblk < 2; ++kblk) {
-        const int key_base = t * AT_KT + kblk * 32;
-        if (key_base < lim_hi) {
-          float e[16];
-          score_exp(kt, kblk, key_base, e);
-          v4i pf;  // 16 int8 probabilities of this lane's row, keys in accumulator order
+      for (int db = 0; db < 4; ++db)
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const unsigned b0 = __float_as_uint(__builtin_fmaf(e[4 * g + 0], rinv, MAGIC));
-            const unsigned b1 = __float_as_uint(__builtin_fmaf(e[4 * g + 1], rinv, MAGIC));
-            const unsigned b2 = __float_as_uint(__builtin_fmaf(e[4 * g + 2], rinv, MAGIC));
-            const unsigned b3 = __float_as_uint(__builtin_fmaf(e[4 * g + 3], rinv, MAGIC));
-            pf[g] = (int)(__builtin_amdgcn_perm(b1, b0, 0x0c0c0400u) | __builtin_amdgcn_perm(b3, b2, 0x04000c0cu));
-          }
+        for (int b = 0; b < 2; ++b) vf[b][db] = *(const v4i*)(vt + (db * 32 + lrow) * AT_VP + b * 32 + lhi * 16);
+      v4i pf[2];  // 16 int8 probabilities of this lane's row per block, keys in accumulator order
 #pragma unroll
-          for (int db = 0; db < 4; ++db) {
-            const v4i vf = *(const v4i*)(vt + (db * 32 + lrow) * AT_VP + kblk * 32 + lhi * 16);
-            o[db] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf, pf, o[db], 0, 0, 0);  // rows of the result = d
-          }
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const unsigned b0 = __float_as_uint(__builtin_fmaf(e[b][4 * g + 0], rinv, MAGIC));
+          const unsigned b1 = __float_as_uint(__builtin_fmaf(e[b][4 * g + 1], rinv, MAGIC));
+          const unsigned b2 = __float_as_uint(__builtin_fmaf(e[b][4 * g + 2], rinv, MAGIC));
+          const unsigned b3 = __float_as_uint(__builtin_fmaf(e[b][4 * g + 3], rinv, MAGIC));
+          pf[b][g] = (int)(__builtin_amdgcn_perm(b1, b0, 0x0c0c0400u) | __builtin_amdgcn_perm(b3, b2, 0x04000c0cu));
         }
-      }
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+          o[db] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf[b][db], pf[b], o[db], 0, 0, 0);  // rows of the result = d
     }
     if (t + 1 < ntiles) stash((t + 1) & 1, true);
     __syncthreads();
