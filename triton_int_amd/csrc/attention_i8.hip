@@ -18,9 +18,8 @@
 // Two passes over the keys of a query block, as the probabilities need the whole row's sum before
 // they can be quantised: pass 1 computes scores and sums exponentials, pass 2 recomputes the
 // scores (K = 128 deep: cheap), forms the int8 probabilities in the MFMA operand layout straight
-// from the accumulator registers and feeds them to the P.V MFMAs.  The order of the keys inside
-// a 32-key block is a free choice (it is the reduction index of P.V): V^T is stored to LDS in
-// the order in which the score accumulators hold the keys, so P never moves between lanes.
+// from the accumulator registers (two half-wave swaps put a row's keys in order) and feeds them
+// to the P.V MFMAs, so P never goes through memory.
 //
 // Workgroup = 4 waves = 128 query rows of one head; a wave owns 32 rows.  K and V^T are staged
 // through LDS in tiles of 64 keys, double-buffered, one barrier per tile.  Causal masking skips
@@ -128,14 +127,7 @@ __global__ __launch_bounds__(256, 2) void attention_i8_kernel(AttnParams p) {
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
         const int q_ = c * 256 + tid;
-        const int vr = q_ >> 2, vc = q_ & 3;
-        // keys 16*vc + 4*w .. +3 (dword w) of their 32-key block are held by the score
-        // accumulators of lane half (w & 1) as register group g = 2*(vc & 1) + (w >> 1):
-        // they go to byte 16*(w & 1) + 4*g of the block
-        char* dst = vt + vr * AT_VP + (vc >> 1) * 32;
-#pragma unroll
-        for (int w = 0; w < 4; ++w)
-          *(int*)(dst + 16 * (w & 1) + 4 * (2 * (vc & 1) + (w >> 1))) = vreg[c][w];
+        *(v4i*)(vt + (q_ >> 2) * AT_VP + (q_ & 3) * 16) = vreg[c];
       }
     }
   };
@@ -246,6 +238,15 @@ __global__ __launch_bounds__(256, 2) void attention_i8_kernel(AttnParams p) {
           const unsigned b3 = __float_as_uint(__builtin_fmaf(e[b][4 * g + 3], rinv, MAGIC));
           pf[b][g] = (int)(__builtin_amdgcn_perm(b1, b0, 0x0c0c0400u) | __builtin_amdgcn_perm(b3, b2, 0x04000c0cu));
         }
+      // The accumulators hold a row's 32 keys of a block as alternate 4-key groups in the two lane
+      // halves; two half-wave swaps give lane half h the keys 16h .. 16h+15 in order, which is how
+      // the MFMA wants its 32-deep operand and how V^T lies in LDS.
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const auto s02 = __builtin_amdgcn_permlane32_swap((unsigned)pf[b][0], (unsigned)pf[b][2], false, false);
+        const auto s13 = __builtin_amdgcn_permlane32_swap((unsigned)pf[b][1], (unsigned)pf[b][3], false, false);
+        pf[b][0] = (int)s02[0]; pf[b][1] = (int)s02[1]; pf[b][2] = (int)s13[0]; pf[b][3] = (int)s13[1];
+      }
 #pragma unroll
       for (int b = 0; b < 2; ++b)
 #pragma unroll
