@@ -246,13 +246,20 @@ def extras(torch, dev):
     of = torch.empty((B, S, D), dtype=torch.float32, device=dev)
     ms = time_region(torch, lambda: bmm.bmm_s8t_s8n_f32t(p, vt, 1.0 / 16129, out=of), 10, 2)
     out["bmm_pv_f32_160x2048x128x2048"] = {"ms": ms, "GBps": 880.8e6 / ms / 1e6, "TOPS": 171.8e9 / ms / 1e9}
-    del q, k, sc, vt, of
+    del sc, of
     # int8 scores -> int8 probabilities (softmax + quantise), 2 B/element
     ms = time_region(torch, lambda: fused.softmax_q(p, 0.05), 10, 2)
     out["softmax_q_160x2048x2048"] = {"ms": ms, "GBps": p.numel() * 2 / ms / 1e6}
     del p
     for v in out.values():
         v["frac_hbm_peak"] = v["GBps"] / HBM_PEAK_GBPS
+    # the same three steps (Q.K^T -> softmax-quantise -> P.V, int8 out) as one kernel: scores and
+    # probabilities stay in registers, so its bound is the VALU work per score, not HBM
+    ctx = torch.empty((B, S, D), dtype=torch.int8, device=dev)
+    for name, q_len in (("full", 0), ("causal", S)):
+        ms = time_region(torch, lambda: fused.attention_i8(q, k, vt, 1e-3, 0.05, 1.0 / 127.0, causal_q_len=q_len, out=ctx), 10, 2)
+        out[f"attention_i8_fused_{name}_160x2048x2048x128"] = {"ms": ms, "scores_per_us": B * S * S / (2 if q_len else 1) / ms / 1e3}
+    del q, k, vt, ctx
     # config 1: one W8A8B8O8Linear 512 x 768 x 768 (launch-latency sized: no roofline claim).  Eager
     # time includes the Python launch path; the graph replay is the kernel alone.
     from triton_int_amd.kernels import linear
