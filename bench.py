@@ -354,6 +354,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU emulation baseline")
     ap.add_argument("--no-extra", action="store_true", help="skip the row-kernel / BMM extras")
+    ap.add_argument("--attention-only", action="store_true",
+                    help="run 3 full and 3 causal launches of the fused attention kernel (40 heads x 2048 x 2048 "
+                         "x 128) and exit: the program profiled for the attention counter summary")
     ap.add_argument("--calib-copy-mb", type=int, default=0,
                     help="before the timed region, run 4 device-to-device copies of this many MiB: a kernel of "
                          "known traffic to scale rocprofv3's FETCH_SIZE / WRITE_SIZE readings with")
@@ -371,6 +374,17 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.attention_only:
+        from triton_int_amd.kernels import fused
+
+        q, k = (torch.randint(-127, 128, (40, 2048, 128), dtype=torch.int8, device=dev) for _ in range(2))
+        vt = torch.randint(-127, 128, (40, 128, 2048), dtype=torch.int8, device=dev)
+        ctx = torch.empty_like(q)
+        for q_len in (0, 2048):
+            for _ in range(3):
+                fused.attention_i8(q, k, vt, 1e-3, 0.05, 1.0 / 127.0, causal_q_len=q_len, out=ctx)
+        torch.cuda.synchronize()
+        return
     layers = build_linear_set(torch, dev)
     # which kernel does each GEMM run on?  (one untimed pass)
     keyed = []
