@@ -67,6 +67,14 @@ def test_decoder_layer_prefill_and_decode_small():
     out = layer(gpu(hidden), _trace=tr)
     assert out.shape == (B, S, H) and out.dtype == torch.float32
     _check_stages(layer, tr, hidden, B, S, causal_q_len=S)
+    # the one-kernel attention forced on for this small two-batch case: same context rows
+    layer.fused_attention_min_queries = 1
+    trf = {}
+    layer(gpu(hidden), _trace=trf)
+    assert trf["scores"] is None
+    diff = (trf["ctx"].int() - tr["ctx"].int()).abs()
+    assert int((diff.amax(dim=-1) > 0).sum()) <= 1 and torch.equal(trf["q"], tr["q"])
+    layer.fused_attention_min_queries = 128
     # decode: 16 new tokens against a cache of T = 80 slots (64 old + 16 new)
     T, Sd = 80, 16
     k_cache = torch.from_numpy(g.integers(-127, 128, size=(B * heads, T, H // heads), dtype=np.int8)).to(DEV)
@@ -78,6 +86,13 @@ def test_decoder_layer_prefill_and_decode_small():
     assert out.shape == (B, Sd, H)
     assert torch.equal(k_cache[:, :T - Sd], k_old[:, :T - Sd]) and torch.equal(vt_cache[:, :, :T - Sd], vt_old[:, :, :T - Sd])
     _check_stages(layer, tr, hidden_d, B, Sd, causal_q_len=Sd)
+    # the same decode step through the one-kernel attention (cache offset T - S in the causal mask)
+    layer.fused_attention_min_queries = 1
+    k2, v2 = k_old.clone(), vt_old.clone()
+    trf = {}
+    layer(gpu(hidden_d), kv_cache=(k2, v2), _trace=trf)
+    diff = (trf["ctx"].int() - tr["ctx"].int()).abs()
+    assert trf["scores"] is None and int((diff.amax(dim=-1) > 0).sum()) <= 1
 
 
 def test_decoder_layer_opt13b_shapes_run():
