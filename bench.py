@@ -233,7 +233,13 @@ def extras(torch, dev):
     xg = torch.randn(8192, 20480, device=dev)
     ms = time_region(torch, lambda: fused.gelu_q(xg, 20.0), 10, 2)
     out["gelu_q_8192x20480"] = {"ms": ms, "GBps": xg.numel() * 5 / ms / 1e6}
-    del xg
+    # per-token dynamic quantisation, fp32 in: 5 B/element; fp16 in: 3 B/element
+    ms = time_region(torch, lambda: fused.quantize_per_token_absmax(xg), 10, 2)
+    out["quantize_per_token_f32_8192x20480"] = {"ms": ms, "GBps": xg.numel() * 5 / ms / 1e6}
+    xh = xg.half()
+    ms = time_region(torch, lambda: fused.quantize_per_token_absmax(xh), 10, 2)
+    out["quantize_per_token_f16_8192x20480"] = {"ms": ms, "GBps": xh.numel() * 3 / ms / 1e6}
+    del xg, xh
     # config 4: attention BMMs, 160 x (2048 x 2048 x 128); HBM-bound (755 MB / 881 MB per call)
     B, S, D = 160, 2048, 128
     q = torch.randint(-127, 128, (B, S, D), dtype=torch.int8, device=dev)

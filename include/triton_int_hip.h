@@ -244,6 +244,19 @@ int ti_attention_i8(const int8_t* q, int64_t q_batch_stride, int64_t q_row_strid
                     int batch, int S, int T, int D,
                     float qk_alpha, float score_scale, float pv_alpha, int causal_q_len, void* stream);
 
+/*
+ * Dynamic per-token activation quantisation, dynamic_quantize_activation_per_token_absmax
+ * (functional/quantization.py:61-67): per row r of x [rows, cols] (fp32 or fp16: x_dtype TI_F32 /
+ * TI_F16, unit column stride, row strides in elements)
+ *     scale[r] = clamp(max_j |x[r,j]|, min = 1e-8) / 127           (rounded to x's dtype per step)
+ *     q[r,j]   = clamp(round_half_even(x[r,j] / scale[r]), -128, 127)
+ * scale_out (rows elements of x's dtype, may be NULL) receives the scales.  x is not modified
+ * (the reference helper overwrites it with the rounded quotients as a side effect).
+ */
+int ti_quantize_per_token_absmax(const void* x, int x_dtype, int64_t x_row_stride,
+                                 int8_t* q, int64_t q_row_stride, void* scale_out,
+                                 int rows, int cols, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -228,3 +228,18 @@ def attention_i8(q, k, vt, qk_alpha, score_scale, pv_alpha, causal_q_len=0, retu
     probs = softmax_q(scores, score_scale, causal_q_len=causal_q_len)
     ctx = bmm_s8t_s8n_s8t(probs, vt, np.float32(pv_alpha))
     return (scores, probs, ctx) if return_all else ctx
+
+
+def quantize_per_token_absmax(t):
+    """dynamic_quantize_activation_per_token_absmax (reference: functional/quantization.py:61-67)
+    restated in numpy, every step in t's dtype (float32 or float16; numpy rounds each float16
+    operation to float16 as torch's elementwise kernels do): returns (q int8, max_val [..., 1])."""
+    dt = t.dtype
+    assert dt in (np.float32, np.float16)
+    max_val = np.abs(t).max(axis=-1, keepdims=True)
+    max_val = np.maximum(max_val.astype(np.float32), np.float32(1e-8)).astype(dt)  # clamp(min=1e-8)
+    max_val = (max_val / dt.type(127)).astype(dt)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        d = (t / max_val).astype(dt)
+    q = np.clip(np.rint(d.astype(np.float32)), -128, 127)
+    return q.astype(np.int8), max_val

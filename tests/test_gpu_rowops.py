@@ -247,3 +247,26 @@ def test_attention_i8_strided_views_and_errors():
         fused.attention_i8(gpu(q3[:, :, :64].copy()), gpu(k3[:, :, :64].copy()), gpu(vt[:, :64].copy()), 1e-3, 0.05, 0.01)
     with pytest.raises(AssertionError):  # score scale too large for the fixed-bound exponent
         fused.attention_i8(gq, gk, gvt, 1e-3, 0.5, 0.01)
+
+
+@pytest.mark.parametrize("rows,cols", [(2048, 5120), (37, 300), (5, 1), (3, 8193), (64, 768), (9, 20480), (2, 40000)])
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_quantize_per_token_absmax(rows, cols, dtype):
+    """Per-token dynamic quantisation: int8 values and scales bit-identical to the oracle's
+    restatement of the reference helper, fp32 and fp16, vector and scalar paths."""
+    fused = _fused()
+    g = rng(rows * 7 + cols)
+    x = (g.standard_normal((rows, cols)) * np.logspace(-3, 2, rows)[:, None]).astype(dtype)
+    x[rows // 2] = dtype(0.25)
+    want_q, want_s = O.quantize_per_token_absmax(x)
+    gx = gpu(x)
+    q, s = fused.quantize_per_token_absmax(gx)
+    assert q.shape == (rows, cols) and s.shape == (rows, 1) and s.dtype == gx.dtype
+    bits = (lambda a: a.view(np.uint16)) if dtype == np.float16 else (lambda a: a)  # cpu() returns fp16 as bits
+    assert np.array_equal(cpu(s), bits(want_s)) and np.array_equal(cpu(q), want_q)
+    assert torch.equal(gx, gpu(x))  # the kernel leaves its input alone
+    # the functional helper keeps the reference's side effect
+    from triton_int_amd.functional.quantization import dynamic_quantize_activation_per_token_absmax
+    q2, s2 = dynamic_quantize_activation_per_token_absmax(gx.view(1, rows, cols))
+    assert q2.shape == (1, rows, cols) and s2.shape == (1, rows, 1)
+    assert np.array_equal(cpu(q2)[0], want_q) and np.array_equal(gx.float().cpu().numpy(), want_q.astype(np.float32))

@@ -165,3 +165,22 @@ def test_softmax_q_vs_torch_softmax():
         lim = (r % q_len) + (cols - q_len) + 1
         p = torch.softmax(torch.from_numpy(xs[r, :lim]).float() * 0.1, dim=-1).mul(127).round().numpy()
         assert np.abs(got[r, :lim] - p).max() <= 1 and np.all(got[r, lim:] == 0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_quantize_per_token_absmax_vs_the_torch_steps(dtype):
+    """The oracle against the five torch calls the reference helper makes
+    (functional/quantization.py:61-67), executed by torch on the CPU in the tensor's dtype."""
+    g = torch.Generator().manual_seed(4)
+    t = (torch.randn((37, 300), generator=g) * torch.logspace(-3, 2, 37).unsqueeze(1)).to(dtype)
+    t[5] = 0.25  # a constant row: every quotient is exactly 127
+    t[6, 7] = 65504.0 if dtype == torch.float16 else 3.0e38
+    x = t.clone()
+    max_val = x.abs().max(dim=-1, keepdim=True)[0]
+    max_val = torch.clamp(max_val, min=1e-8) / 127
+    x.div_(max_val).round_().clamp_(-128, 127)
+    want_q, want_s = x.to(torch.int8).numpy(), max_val.numpy()
+    got_q, got_s = O.quantize_per_token_absmax(t.numpy())
+    assert got_s.dtype == want_s.dtype and np.array_equal(got_s, want_s)
+    assert np.array_equal(got_q, want_q)
+    assert np.abs(got_q[5]).max() == 127 and set(np.unique(got_q[5])) == {127}

@@ -59,6 +59,13 @@ def dynamic_quantize_activation_per_tensor_absmax(t):
 
 @torch.no_grad()
 def dynamic_quantize_activation_per_token_absmax(t):
+    if t.is_cuda and t.dtype in (torch.float32, torch.float16):
+        # one HIP kernel instead of five torch passes; the reference helper also leaves the rounded
+        # quotients in `t` (functional/quantization.py:65), kept here for callers that rely on it
+        from ..kernels.fused import quantize_per_token_absmax
+        q, scale = quantize_per_token_absmax(t)
+        t.copy_(q)
+        return q, scale
     scale = torch.clamp(_absmax_scale(t, dim=-1), min=1e-8) / _QMAX
     t.div_(scale).round_().clamp_(-128, 127)
     return t.to(torch.int8), scale

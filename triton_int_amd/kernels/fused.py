@@ -167,3 +167,25 @@ def attention_i8(q, k, vt, qk_alpha, score_scale, pv_alpha, causal_q_len=0, out=
                                      int(causal_q_len), L.current_stream(q.device))
     L.check(rc, "ti_attention_i8")
     return out
+
+
+def quantize_per_token_absmax(t):
+    """Dynamic per-token quantisation of fp32 / fp16 activations [..., cols]: returns
+    (q int8 [..., cols], max_val [..., 1] in t's dtype) with max_val = clamp(absmax, 1e-8) / 127
+    and q = clamp(round(t / max_val), -128, 127), bit-identical to
+    dynamic_quantize_activation_per_token_absmax (reference: functional/quantization.py:61-67).
+    Unlike that helper it leaves `t` untouched."""
+    L.require_cuda(t)
+    assert t.dtype in (torch.float32, torch.float16), "activations must be fp32 or fp16"
+    cols = t.shape[-1]
+    x2 = t.reshape(-1, cols)
+    if x2.stride(1) != 1:
+        x2 = x2.contiguous()
+    rows = x2.shape[0]
+    q = torch.empty((rows, cols), dtype=torch.int8, device=t.device)
+    scale = torch.empty((rows, 1), dtype=t.dtype, device=t.device)
+    with L.on_device(t.device):
+        rc = L.lib().ti_quantize_per_token_absmax(L.ptr(x2), L.TORCH_TO_DT[t.dtype], x2.stride(0), L.ptr(q), cols,
+                                                  L.ptr(scale), rows, cols, L.current_stream(t.device))
+    L.check(rc, "ti_quantize_per_token_absmax")
+    return q.view(t.shape), scale.view(*t.shape[:-1], 1)
