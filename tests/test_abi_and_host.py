@@ -97,3 +97,31 @@ def test_from_float_algebra_on_cpu():
     assert m.bias.dtype == torch.int32 and torch.allclose(m.b, bs / 0.05)
     assert abs(float(BMM_S8T_S8N_S8T.from_scale(0.02, 0.03, 0.6).a) - 0.001) < 1e-9
     assert abs(float(BMM_S8T_S8N_F32T.from_scale(0.5, 0.25).a) - 0.125) < 1e-9
+
+
+def test_torch_ops_are_registered_with_meta_implementations():
+    """torch.ops.triton_op.* (the namespace the reference registers under, kernels/__init__.py:5)
+    exist and propagate shapes and dtypes on meta tensors, which is what tracing needs."""
+    import torch
+    from triton_int_amd.kernels import _ops
+
+    assert len(_ops.registered) == len(_ops._OPS)
+    m = lambda shape, dt=torch.int8: torch.empty(shape, dtype=dt, device="meta")
+    s = m((), torch.float32)
+    ops = torch.ops.triton_op
+    for name in ("linear_a8_w8_b8_o8", "linear_relu_a8_w8_b8_o8", "linear_a8_w8_bfp32_ofp32_GeLu_Q"):
+        bias = m(32, torch.float32 if "GeLu" in name else torch.int8)
+        y = getattr(ops, name)(m((3, 5, 64)), m((32, 64)), bias, s, s)
+        assert y.shape == (3, 5, 32) and y.dtype == torch.int8 and y.device.type == "meta"
+    assert ops.linear_a8_w8_b32_o32(m((7, 64)), m((32, 64)), None).dtype == torch.int32
+    assert ops.linear_a8_w8_bfp32_ofp32(m((7, 64)), m((32, 64)), m(32, torch.float32), s, s).dtype == torch.float32
+    assert ops.bmm_s8t_s8n_s8t(m((2, 3, 16)), m((2, 9, 16)), 0.5).shape == (2, 3, 9)
+    assert ops.bmm_s8t_s8t_s32t(m((2, 3, 16)), m((2, 16, 9))).shape == (2, 3, 9)
+    assert ops.bmm_s8t_s8n_f32t(m((2, 3, 16)), m((2, 9, 16)), 0.5).dtype == torch.float32
+    assert ops.layer_norm_fwd_fused_single_pass_q(m((4, 8), torch.float32), m(8, torch.float32), None, 1e-5).dtype == torch.int8
+    r, q = ops.dq_add_layernorm_q(m((4, 8), torch.int32), 0.1, m((4, 8), torch.float32), m(8, torch.float32), m(8, torch.float32), 1e-5)
+    assert r.dtype == torch.float32 and q.dtype == torch.int8 and q.shape == (4, 8)
+    assert ops.softmax_q(m((2, 4, 16)), 0.05).shape == (2, 4, 16)
+    assert ops.attention_i8(m((2, 4, 128)), m((2, 16, 128)), m((2, 128, 16)), 1e-3, 0.05, 0.01, 4).shape == (2, 4, 128)
+    q8, sc = ops.quantize_per_token_absmax(m((3, 5, 16), torch.float16))
+    assert q8.shape == (3, 5, 16) and sc.shape == (3, 5, 1) and sc.dtype == torch.float16

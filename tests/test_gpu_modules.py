@@ -157,3 +157,23 @@ def test_baseline_config4_attention_bmms_opt13b_shapes():
     s12 = bmm_s8t_s8n_s32t(probs, gpu((v1 + v2).astype(np.int8)))
     s1 = bmm_s8t_s8n_s32t(probs, gpu(v1)); s2 = bmm_s8t_s8n_s32t(probs, gpu(v2))
     assert torch.equal(s12, s1 + s2)
+
+
+def test_registered_torch_ops_dispatch_and_trace():
+    """torch.ops.triton_op.* run the same kernels as the launchers, and a function that calls them
+    can be captured as one graph (torch.compile with the `eager` backend: tracing only)."""
+    from triton_int_amd.kernels import linear
+    g = rng(21)
+    a, w, b = rand_i8(g, 48, 64), rand_i8(g, 32, 64), rand_i8(g, 32)
+    ga, gw, gb = gpu(a), gpu(w), gpu(b)
+    sa, sb = torch.tensor(0.003, device=DEV), torch.tensor(0.02, device=DEV)
+    want = linear.linear_a8_w8_b8_o8(ga, gw, gb, sa, sb)
+    assert torch.equal(torch.ops.triton_op.linear_a8_w8_b8_o8(ga, gw, gb, sa, sb), want)
+    assert np.array_equal(cpu(want), O.linear_a8_w8_b8_o8(a, w, b, np.float32(0.003), np.float32(0.02)))
+
+    def f(x):
+        y = torch.ops.triton_op.linear_relu_a8_w8_b8_o8(x, gw, gb, sa, sb)
+        return torch.ops.triton_op.gelu_q(y.float(), 2.0)
+
+    compiled = torch.compile(f, backend="eager", fullgraph=True)
+    assert torch.equal(compiled(ga), f(ga))
