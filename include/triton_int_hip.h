@@ -222,6 +222,18 @@ int ti_transpose_i8(const int8_t* src, int64_t src_row_stride, int8_t* dst, int6
                     int rows, int cols, void* stream);
 
 /*
+ * Appends S new positions to an int8 KV cache in one launch: K [S, heads*D] (row stride
+ * k_src_row_stride) is copied to k_dst[h][s][d] = k_dst + h * k_head_stride + s * D + d (k_dst points at
+ * the first new slot of head 0 in a [heads, T, D] cache, k_head_stride = T * D), and V [S, heads*D]
+ * is transposed into vt_dst[(h*D + d) * vt_row_stride + s] (vt_dst points at the first new column
+ * of a [heads*D, T] cache, vt_row_stride = T).  D % 16 == 0.  The reference's callers do both
+ * steps with torch indexing; ti_transpose_i8 alone covers the prefill case without a cache.
+ */
+int ti_kv_append_i8(const int8_t* k_src, int64_t k_src_row_stride, const int8_t* v_src, int64_t v_src_row_stride,
+                    int8_t* k_dst, int64_t k_head_stride, int8_t* vt_dst, int64_t vt_row_stride,
+                    int S, int heads, int D, void* stream);
+
+/*
  * One attention block without the score round trip through memory:
  *     scores = q8(qk_alpha * (q . k^T))                    (bmm_s8t_s8n_s8t, kernels/bmm.py:576-612)
  *     probs  = round_half_even(127 * softmax(scores * score_scale)), causal mask as ti_softmax_q

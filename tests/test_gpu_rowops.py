@@ -270,3 +270,29 @@ def test_quantize_per_token_absmax(rows, cols, dtype):
     q2, s2 = dynamic_quantize_activation_per_token_absmax(gx.view(1, rows, cols))
     assert q2.shape == (1, rows, cols) and s2.shape == (1, rows, 1)
     assert np.array_equal(cpu(q2)[0], want_q) and np.array_equal(gx.float().cpu().numpy(), want_q.astype(np.float32))
+
+
+@pytest.mark.parametrize("S,heads,D,T", [(16, 40, 128, 2048), (48, 4, 128, 80), (70, 3, 64, 100), (1, 2, 16, 5)])
+def test_kv_append_i8(S, heads, D, T):
+    """Pure data movement: K rows into a head-major cache, V transposed into V^T columns; the
+    checker is numpy indexing.  Sources are column slices of a wider matrix, as in the layer."""
+    fused = _fused()
+    g = rng(S + heads * D + T)
+    H = heads * D
+    qkv = g.integers(-128, 128, size=(S, 3 * H), dtype=np.int8)
+    k_cache = g.integers(-128, 128, size=(heads, T, D), dtype=np.int8)
+    vt_cache = g.integers(-128, 128, size=(heads, D, T), dtype=np.int8)
+    want_k, want_vt = k_cache.copy(), vt_cache.copy()
+    want_k[:, T - S:, :] = qkv[:, H:2 * H].reshape(S, heads, D).transpose(1, 0, 2)
+    want_vt[:, :, T - S:] = qkv[:, 2 * H:].reshape(S, heads, D).transpose(1, 2, 0)
+    gq, gk, gv = gpu(qkv), gpu(k_cache), gpu(vt_cache)
+    fused.kv_append_i8(gq[:, H:2 * H], gq[:, 2 * H:], gk, gv)
+    assert np.array_equal(cpu(gk), want_k) and np.array_equal(cpu(gv), want_vt)
+    # unaligned sources (a slice that starts at an odd column) take the byte path
+    wide = g.integers(-128, 128, size=(S, 2 * H + 1), dtype=np.int8)
+    gw = gpu(wide)
+    gk, gv = gpu(k_cache), gpu(vt_cache)
+    fused.kv_append_i8(gw[:, 1:H + 1], gw[:, H + 1:], gk, gv)
+    want_k[:, T - S:, :] = wide[:, 1:H + 1].reshape(S, heads, D).transpose(1, 0, 2)
+    want_vt[:, :, T - S:] = wide[:, H + 1:].reshape(S, heads, D).transpose(1, 2, 0)
+    assert np.array_equal(cpu(gk), want_k) and np.array_equal(cpu(gv), want_vt)

@@ -523,6 +523,60 @@ __global__ __launch_bounds__(256) void transpose_i8_kernel(const int8_t* __restr
   }
 }
 
+// KV-cache append of S new positions in one launch: blockIdx.z == 0 transposes V [S, heads*D] into
+// columns of V^T [heads*D, T] (the kernel above), blockIdx.z == 1 copies K [S, heads*D] into the
+// head-major cache [heads, T, D], 16 bytes per thread (D % 16 == 0).
+__global__ __launch_bounds__(256) void kv_append_i8_kernel(const int8_t* __restrict__ k_src, int64_t k_rs,
+                                                           const int8_t* __restrict__ v_src, int64_t v_rs,
+                                                           int8_t* __restrict__ k_dst, int64_t k_head_stride,
+                                                           int8_t* __restrict__ vt_dst, int64_t vt_rs, int S, int H, int D,
+                                                           int vec) {
+  if (blockIdx.z == 0) {
+    __shared__ __attribute__((aligned(16))) int8_t tile[TR_TILE][TR_PITCH];
+    const int t = threadIdx.x;
+    const int r0 = blockIdx.y * TR_TILE, c0 = blockIdx.x * TR_TILE;
+    {
+      const int r = t >> 2, cc = (t & 3) * 16;
+      unsigned w[4] = {0u, 0u, 0u, 0u};
+      if (r0 + r < S && c0 + cc < H) {  // H % 16 == 0: a chunk is inside or outside
+        const int8_t* sp = v_src + (int64_t)(r0 + r) * v_rs + c0 + cc;
+        if (vec) {
+          const v4u v = *(const v4u*)sp;
+          w[0] = v[0]; w[1] = v[1]; w[2] = v[2]; w[3] = v[3];
+        } else {
+          for (int i = 0; i < 16; ++i) w[i >> 2] |= (unsigned)(uint8_t)sp[i] << ((i & 3) * 8);
+        }
+      }
+#pragma unroll
+      for (int g = 0; g < 4; ++g) *(unsigned*)&tile[r][cc + 4 * g] = w[g];
+    }
+    __syncthreads();
+    const int c = t >> 2, rr = (t & 3) * 16;
+    if (c0 + c >= H) return;
+    unsigned w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 16; ++i) w[i >> 2] |= (unsigned)(uint8_t)tile[rr + i][c] << ((i & 3) * 8);
+    int8_t* dp = vt_dst + (int64_t)(c0 + c) * vt_rs + r0 + rr;
+    if (vec && r0 + rr + 16 <= S) {
+      *(v4u*)dp = (v4u){w[0], w[1], w[2], w[3]};
+    } else {
+      for (int i = 0; i < 16; ++i)
+        if (r0 + rr + i < S) dp[i] = (int8_t)(w[i >> 2] >> ((i & 3) * 8));
+    }
+  } else {
+    const int t = threadIdx.x;
+    const int r = blockIdx.y * TR_TILE + (t >> 2), c = blockIdx.x * TR_TILE + (t & 3) * 16;
+    if (r >= S || c >= H) return;
+    const int8_t* sp = k_src + (int64_t)r * k_rs + c;
+    int8_t* dp = k_dst + (int64_t)(c / D) * k_head_stride + (int64_t)r * D + (c % D);
+    if (vec) {
+      *(v4u*)dp = *(const v4u*)sp;
+    } else {
+      for (int i = 0; i < 16; ++i) dp[i] = sp[i];
+    }
+  }
+}
+
 }  // namespace ti
 
 extern "C" {
@@ -633,6 +687,29 @@ int ti_transpose_i8(const int8_t* src, int64_t src_row_stride, int8_t* dst, int6
   ti::transpose_i8_kernel<<<grid, dim3(256), 0, (hipStream_t)stream>>>(src, src_row_stride, dst, dst_row_stride, rows,
                                                                     cols, vec_src, vec_dst);
   return ti::launch_status("transpose_i8_kernel");
+}
+
+int ti_kv_append_i8(const int8_t* k_src, int64_t k_src_row_stride, const int8_t* v_src, int64_t v_src_row_stride,
+                    int8_t* k_dst, int64_t k_head_stride, int8_t* vt_dst, int64_t vt_row_stride, int S, int heads, int D,
+                    void* stream) {
+  if (S < 0 || heads < 0 || D < 0) return ti::fail(TI_E_SHAPE, "negative size");
+  if (S == 0 || heads == 0 || D == 0) return TI_OK;
+  if (!k_src || !v_src || !k_dst || !vt_dst) return ti::fail(TI_E_NULL, "k_src, v_src, k_dst and vt_dst are required");
+  if (D & 15) return ti::fail(TI_E_SHAPE, "head dimension %d must be a multiple of 16", D);
+  const int64_t H = (int64_t)heads * D;
+  if (H > 0x7fffffff) return ti::fail(TI_E_SHAPE, "heads * D too large");
+  if (k_src_row_stride < H || v_src_row_stride < H || vt_row_stride < S || k_head_stride < (int64_t)S * D)
+    return ti::fail(TI_E_STRIDE, "strides must cover the rows they step over");
+  int rc = ti::check_device();
+  if (rc != TI_OK) return rc;
+  const int vec = ((((uintptr_t)k_src) | ((uintptr_t)v_src) | ((uintptr_t)k_dst) | ((uintptr_t)vt_dst) |
+                    (uintptr_t)k_src_row_stride | (uintptr_t)v_src_row_stride | (uintptr_t)k_head_stride |
+                    (uintptr_t)vt_row_stride) & 15) == 0;
+  dim3 grid((unsigned)((H + ti::TR_TILE - 1) / ti::TR_TILE), (unsigned)((S + ti::TR_TILE - 1) / ti::TR_TILE), 2);
+  if (grid.y > 65535) return ti::fail(TI_E_SHAPE, "more than 65535 * 64 positions");
+  ti::kv_append_i8_kernel<<<grid, dim3(256), 0, (hipStream_t)stream>>>(k_src, k_src_row_stride, v_src, v_src_row_stride, k_dst,
+                                                                    k_head_stride, vt_dst, vt_row_stride, S, (int)H, D, vec);
+  return ti::launch_status("kv_append_i8_kernel");
 }
 
 }  // extern "C"

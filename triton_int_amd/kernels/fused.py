@@ -189,3 +189,21 @@ def quantize_per_token_absmax(t):
                                                   L.ptr(scale), rows, cols, L.current_stream(t.device))
     L.check(rc, "ti_quantize_per_token_absmax")
     return q.view(t.shape), scale.view(*t.shape[:-1], 1)
+
+
+def kv_append_i8(k_new, v_new, k_cache, vt_cache):
+    """Write S new positions into the last S slots of an int8 KV cache with one launch.
+    k_new, v_new: int8 [S, heads*D] (unit column stride; e.g. column slices of a fused q/k/v
+    projection); k_cache int8 [heads, T, D]; vt_cache int8 [heads, D, T].  Replaces
+    `k_cache[:, T-S:, :] = k_new.view(S, heads, D).transpose(0, 1)` and the V transpose."""
+    L.require_cuda(k_new, v_new, k_cache, vt_cache)
+    heads, T, D = k_cache.shape
+    S, H = k_new.shape
+    assert H == heads * D and tuple(v_new.shape) == (S, H) and tuple(vt_cache.shape) == (heads, D, T) and S <= T
+    assert k_new.dtype == v_new.dtype == k_cache.dtype == vt_cache.dtype == torch.int8
+    assert k_new.stride(1) == 1 and v_new.stride(1) == 1 and k_cache.is_contiguous() and vt_cache.is_contiguous()
+    with L.on_device(k_new.device):
+        rc = L.lib().ti_kv_append_i8(L.ptr(k_new), k_new.stride(0), L.ptr(v_new), v_new.stride(0),
+                                     k_cache.data_ptr() + (T - S) * D, T * D, vt_cache.data_ptr() + (T - S), T,
+                                     S, heads, D, L.current_stream(k_new.device))
+    L.check(rc, "ti_kv_append_i8")

@@ -23,7 +23,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels.bmm import bmm_s8t_s8n_s8t
-from ..kernels.fused import attention_i8, softmax_q, transpose_i8
+from ..kernels.fused import attention_i8, kv_append_i8, softmax_q, transpose_i8
 from ..kernels.linear import linear_group_a8_w8_b8_o8
 from .fused import DQ_Add_LayerNorm_Q, LayerNormQ, W8A8BFP32OFP32_GeLu_Q
 from .linear import W8A8B8O8Linear, W8A8B32O32LinearWithoutScaling, W8A8BFP32OFP32Linear
@@ -125,14 +125,21 @@ class W8A8OPTDecoderLayer(torch.nn.Module):
         if kv_cache is None:
             k_all = k_new
             vt_all = torch.empty((B * self.heads, self.head_dim, S), dtype=torch.int8, device=hidden.device)
+            # V^T of every head of a batch in one transpose: [S, heads*D] -> [heads*D, S]
+            for b in range(B):
+                transpose_i8(v[b], out=vt_all[b * self.heads:(b + 1) * self.heads].view(H, S))
         else:
+            # the new K rows and V^T columns go into the last S slots of the cache, one launch per batch
             k_all, vt_all = kv_cache
-            T = k_all.shape[1]
-            k_all[:, T - S:, :] = k_new
-        T = vt_all.shape[2]
-        # V^T of every head of a batch in one transpose: [S, heads*D] -> the last S columns of [heads*D, T]
-        for b in range(B):
-            transpose_i8(v[b], out=vt_all[b * self.heads:(b + 1) * self.heads].view(H, T)[:, T - S:])
+            if k_all.is_contiguous() and vt_all.is_contiguous() and self.head_dim % 16 == 0:
+                for b in range(B):
+                    hs = slice(b * self.heads, (b + 1) * self.heads)
+                    kv_append_i8(qkv[b, :, H:2 * H], v[b], k_all[hs], vt_all[hs])
+            else:
+                T = k_all.shape[1]
+                k_all[:, T - S:, :] = k_new
+                for b in range(B):
+                    transpose_i8(v[b], out=vt_all[b * self.heads:(b + 1) * self.heads].view(H, T)[:, T - S:])
         mark("kv_append_v_transpose")
         T = k_all.shape[1]
         ctx = torch.empty((B, S, H), dtype=torch.int8, device=hidden.device)
