@@ -1,5 +1,6 @@
 // rowops.hip — HBM-bound row kernels for gfx950: LayerNorm -> int8, dequant + residual add +
-// LayerNorm -> int8, and tanh-GELU -> int8.
+// LayerNorm -> int8, tanh-GELU -> int8, softmax -> int8 probabilities, int8 transpose and
+// KV-cache append.
 //
 // Replaces kernel_layer_norm_fwd_fused_single_pass_q (kernels/fused.py:235-382 of
 // zhanglei1172/triton_int), supplies the native dq_add_layernorm_q the reference only emulates
