@@ -360,6 +360,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU emulation baseline")
     ap.add_argument("--no-extra", action="store_true", help="skip the row-kernel / BMM extras")
+    ap.add_argument("--decode-gemm-only", action="store_true",
+                    help="run 24 launches of the M=16 decode GEMM 20480 x 5120 (int8 out, weights rotated through "
+                         "6 matrices) and exit: the program profiled for the decode GEMM counter summary")
     ap.add_argument("--attention-only", action="store_true",
                     help="run 3 full and 3 causal launches of the fused attention kernel (40 heads x 2048 x 2048 "
                          "x 128) and exit: the program profiled for the attention counter summary")
@@ -380,6 +383,17 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.decode_gemm_only:
+        from triton_int_amd.kernels import linear
+
+        ws = [torch.randint(-127, 128, (20480, 5120), dtype=torch.int8, device=dev) for _ in range(6)]
+        x = torch.randint(-127, 128, (16, 5120), dtype=torch.int8, device=dev)
+        b8 = torch.randint(-127, 128, (20480,), dtype=torch.int8, device=dev)
+        al, be = torch.tensor(0.002, device=dev), torch.tensor(0.01, device=dev)
+        for i in range(24):
+            linear.linear_a8_w8_b8_o8(x, ws[i % 6], b8, al, be)
+        torch.cuda.synchronize()
+        return
     if args.attention_only:
         from triton_int_amd.kernels import fused
 

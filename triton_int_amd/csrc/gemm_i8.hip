@@ -1407,11 +1407,15 @@ __global__ __launch_bounds__(512, UU ? 2 : 4) void gemm_skinny_kernel(GemmParams
 // a time, three chunks deep, and shared by the 8 consumer waves; a barrier per chunk hands them
 // over.  Operand fragments then come from LDS: rows 4..15 of the 16-row MFMA operand repeat rows
 // 0..3 (their results are dropped), so no K split and no reduction between waves is needed.
-constexpr int R4_NW = 8, R4_RG = 4, R4_KC = 1024, R4_PITCH = R4_KC + 16, R4_NST = 3, R4_XB = 3, R4_UMAX = 4;
+// LDS row pitches: activation rows are read 16 rows x 4 chunks at a time (pitch = 4 banks mod 64: the
+// 16 rows of a quarter wave hit 64 different banks); a weight job's 4 rows are read 4 rows x 4 chunks
+// with every address shared by 4 lanes (pitch = 16 banks mod 64: 16 different bank groups).
+constexpr int R4_NW = 8, R4_RG = 4, R4_KC = 1024, R4_PITCH = R4_KC + 16, R4_WPITCH = R4_KC + 64, R4_NST = 3, R4_XB = 3,
+              R4_UMAX = 4;
 
 template <int OUTCLS>
 __global__ __launch_bounds__((R4_NW + 1) * 64) void gemm_rows4_kernel(GemmParams p) {
-  constexpr int STAGE = R4_RG * R4_PITCH;  // one job: 4 rows x 1 KB (+ padding against bank conflicts)
+  constexpr int STAGE = R4_RG * R4_WPITCH;  // one job: 4 rows x 1 KB (+ padding against bank conflicts)
   constexpr int XBUF = 16 * R4_PITCH;
   __shared__ __attribute__((aligned(16))) char lds[R4_XB * XBUF + R4_NW * R4_NST * STAGE];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -1462,7 +1466,7 @@ __global__ __launch_bounds__((R4_NW + 1) * 64) void gemm_rows4_kernel(GemmParams
   const unsigned ring = lds_base + R4_XB * XBUF + wave * (R4_NST * STAGE);
   char* ring_p = lds + R4_XB * XBUF + wave * (R4_NST * STAGE);
   const int r16 = lane & 15, c4 = lane >> 4;
-  const int w_lane = (r16 & (R4_RG - 1)) * R4_PITCH + c4 * 16;  // rows 4..15 of the operand repeat rows 0..3
+  const int w_lane = (r16 & (R4_RG - 1)) * R4_WPITCH + c4 * 16;  // rows 4..15 of the operand repeat rows 0..3
   const int x_lane = r16 * R4_PITCH + c4 * 16;
   const EpiCtx e = make_epi(p, bz);
   constexpr int ESZ = OUTCLS == OUT8 ? 1 : (OUTCLS == OUT32 ? 4 : 2);
@@ -1487,7 +1491,7 @@ __global__ __launch_bounds__((R4_NW + 1) * 64) void gemm_rows4_kernel(GemmParams
       const unsigned dst = ring + (j % R4_NST) * STAGE;
 #pragma unroll
       for (int r = 0; r < R4_RG; ++r)
-        dma16_to_lds(rW, in ? min(row0 + r, p.N - 1) * ldb + kl : OOB, k0, dst + r * R4_PITCH);
+        dma16_to_lds(rW, in ? min(row0 + r, p.N - 1) * ldb + kl : OOB, k0, dst + r * R4_WPITCH);
     };
     v4i acc[R4_UMAX];
 #pragma unroll
