@@ -227,6 +227,15 @@ __device__ __forceinline__ void dma16_to_lds(v4i rsrc, int voff, int soff, unsig
                : "memory");
 }
 
+// the same, non-temporal, for data that is read exactly once (the decode kernel's weight stream:
+// 7 % shorter launches than with the default cache policy)
+__device__ __forceinline__ void dma16_to_lds_stream(v4i rsrc, int voff, int soff, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen nt lds"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
+               : "memory");
+}
+
 // wait until at most N of this wave's buffer loads are outstanding and its LDS reads are done,
 // then meet the other waves of the workgroup
 template <int N>
@@ -1025,6 +1034,8 @@ __global__ __launch_bounds__((WAVES_M * WAVES_N + PW) * 64) void gemm_mfma_ws_ke
     const int OOB = (int)0x80000000;
     v4i rA, rB;
     int i_issue = 0, k_issue = 0, st_issue = 0, kt_left = 0;
+    // one column of tiles: every byte of A is read exactly once, so it need not stay in the caches
+    const bool a_once = p.tiles_n == 1;
     auto aim = [&](int i) {
       kt_left = KT;
       k_issue = 0;
@@ -1042,9 +1053,15 @@ __global__ __launch_bounds__((WAVES_M * WAVES_N + PW) * 64) void gemm_mfma_ws_ke
       }
     };
     auto issue_ktile = [&]() {
+      if (a_once) {
 #pragma unroll
-      for (int d = 0; d < A_IT; ++d)
-        dma16_to_lds(rA, (k_issue < la.klim[d]) ? la.voff[d] : OOB, k_issue, wave_slot + st_issue * STAGE + d * NTP * 16);
+        for (int d = 0; d < A_IT; ++d)
+          dma16_to_lds_stream(rA, (k_issue < la.klim[d]) ? la.voff[d] : OOB, k_issue, wave_slot + st_issue * STAGE + d * NTP * 16);
+      } else {
+#pragma unroll
+        for (int d = 0; d < A_IT; ++d)
+          dma16_to_lds(rA, (k_issue < la.klim[d]) ? la.voff[d] : OOB, k_issue, wave_slot + st_issue * STAGE + d * NTP * 16);
+      }
 #pragma unroll
       for (int d = 0; d < B_IT; ++d)
         dma16_to_lds(rB, (k_issue < lb.klim[d]) ? lb.voff[d] : OOB, k_issue,
@@ -1491,7 +1508,7 @@ __global__ __launch_bounds__((R4_NW + 1) * 64) void gemm_rows4_kernel(GemmParams
       const unsigned dst = ring + (j % R4_NST) * STAGE;
 #pragma unroll
       for (int r = 0; r < R4_RG; ++r)
-        dma16_to_lds(rW, in ? min(row0 + r, p.N - 1) * ldb + kl : OOB, k0, dst + r * R4_WPITCH);
+        dma16_to_lds_stream(rW, in ? min(row0 + r, p.N - 1) * ldb + kl : OOB, k0, dst + r * R4_WPITCH);
     };
     v4i acc[R4_UMAX];
 #pragma unroll
