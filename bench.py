@@ -240,6 +240,17 @@ def extras(torch, dev):
     ms = time_region(torch, lambda: fused.quantize_per_token_absmax(xh), 10, 2)
     out["quantize_per_token_f16_8192x20480"] = {"ms": ms, "GBps": xh.numel() * 3 / ms / 1e6}
     del xg, xh
+    # floating-point LayerNorm and the skip variant with both outputs (fp16: 4 and 8 B/element;
+    # fp32: 8 and 16 B/element), 16384 x 5120 so that the fp16 tensors exceed the MALL as well
+    for dt, name, eb in ((torch.float16, "f16", 2), (torch.float32, "f32", 4)):
+        xl = torch.randn(16384, 5120, device=dev).to(dt)
+        sk = torch.randn(16384, 5120, device=dev).to(dt)
+        gl, bl = (torch.randn(5120, device=dev) * 0.1 + 1).to(dt), (torch.randn(5120, device=dev) * 0.1).to(dt)
+        ms = time_region(torch, lambda: fused.layer_norm_fwd_fused_single_pass(xl, gl, bl, 1e-5), 10, 2)
+        out[f"layer_norm_{name}_16384x5120"] = {"ms": ms, "GBps": xl.numel() * 2 * eb / ms / 1e6}
+        ms = time_region(torch, lambda: fused.skip_layer_norm_fwd_fused_single_pass2(xl, sk, gl, bl, 1e-5), 10, 2)
+        out[f"skip_layer_norm2_{name}_16384x5120"] = {"ms": ms, "GBps": xl.numel() * 4 * eb / ms / 1e6}
+        del xl, sk
     # config 4: attention BMMs, 160 x (2048 x 2048 x 128); HBM-bound (755 MB / 881 MB per call)
     B, S, D = 160, 2048, 128
     q = torch.randint(-127, 128, (B, S, D), dtype=torch.int8, device=dev)

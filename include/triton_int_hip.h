@@ -269,6 +269,23 @@ int ti_quantize_per_token_absmax(const void* x, int x_dtype, int64_t x_row_strid
                                  int8_t* q, int64_t q_row_stride, void* scale_out,
                                  int rows, int cols, void* stream);
 
+/*
+ * Floating-point LayerNorm / RMSNorm over the rows of x [rows, cols], with the optional skip
+ * (residual) add: layer_norm_fwd_fused_single_pass (kernels/fused.py:385-532),
+ * skip_layer_norm_fwd_fused_single_pass (kernels/fused.py:535-693) and
+ * skip_layer_norm_fwd_fused_single_pass2 (kernels/fused.py:696-862).  All tensors share one dtype
+ * (TI_F32 / TI_F16 / TI_BF16), unit column stride, row strides in elements.
+ *     a = f32(x); mean = sum(a)/cols (0 when rms != 0); var = sum((a-mean)^2)/cols
+ *     out      = T( ((a - mean) / sqrt(var + eps)) * f32(gamma) [+ f32(beta)] )      (beta may be NULL)
+ *     skip_out = T( f32(out) + f32(skip) )
+ * out alone: the plain LayerNorm; skip + skip_out alone: the first skip variant; all three: the
+ * second.  skip and skip_out are both NULL or both given.
+ */
+int ti_layernorm_fp(const void* x, int64_t x_row_stride, const void* skip, int64_t skip_row_stride, int dtype,
+                    const void* gamma, const void* beta, float eps, int rms,
+                    void* out, int64_t out_row_stride, void* skip_out, int64_t skip_out_row_stride,
+                    int rows, int cols, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -243,3 +243,51 @@ def quantize_per_token_absmax(t):
         d = (t / max_val).astype(dt)
     q = np.clip(np.rint(d.astype(np.float32)), -128, 127)
     return q.astype(np.int8), max_val
+
+
+def _round_fp(v32, kind):
+    """float32 values rounded (half to even) to `kind` in {"f32", "f16", "bf16"}, returned as float32."""
+    v32 = np.asarray(v32, dtype=np.float32)
+    if kind == "f32":
+        return v32
+    if kind == "f16":
+        with np.errstate(over="ignore"):  # beyond 65504 -> inf, as the hardware conversion gives
+            return v32.astype(np.float16).astype(np.float32)
+    assert kind == "bf16"
+    u = v32.view(np.uint32).astype(np.uint64)
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+    r = np.where(nan, (u | 0x400000) & 0xFFFF0000, r).astype(np.uint32)
+    return r.view(np.float32)
+
+
+def layer_norm_fp(x, weight, bias, eps, rms=False, skip=None, kind="f32"):
+    """layer_norm_fwd_fused_single_pass / skip_layer_norm_fwd_fused_single_pass(2)
+    (reference: kernels/fused.py:385-862).  All tensors are float32 arrays holding values
+    representable in `kind` ("f32", "f16", "bf16"); returns (out, skip_out) the same way
+    (skip_out is None without skip).  Statistics: the row's mean and biased variance evaluated in
+    float64 and rounded to float32 (what any fp32 summation order approximates to a few ulps);
+    normalisation: ((a - mean) * rstd) * w (+ b), each step rounded to float32
+    (kernels/fused.py:473-477); out rounded to `kind`, skip_out = round(out + skip)
+    (kernels/fused.py:630-640).  fp16 callers raise eps to 1.6e-5 first (kernels/fused.py:502-503)."""
+    shape = x.shape
+    a = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, shape[-1])
+    w = np.asarray(weight, dtype=np.float32)
+    a64 = a.astype(np.float64)
+    if rms:
+        mean = np.zeros((a.shape[0], 1), np.float32)
+        var = (a64 * a64).mean(axis=1, keepdims=True).astype(np.float32)
+    else:
+        mean64 = a64.mean(axis=1, keepdims=True)
+        mean = mean64.astype(np.float32)
+        var = ((a64 - mean64) ** 2).mean(axis=1, keepdims=True).astype(np.float32)
+    rstd = (np.float32(1.0) / np.sqrt(var + np.float32(eps), dtype=np.float32)).astype(np.float32)
+    o = ((a - mean) * rstd).astype(np.float32) * w
+    if bias is not None:
+        o = o + np.asarray(bias, dtype=np.float32)
+    out = _round_fp(o.astype(np.float32), kind)
+    skip_out = None
+    if skip is not None:
+        s = np.ascontiguousarray(skip, dtype=np.float32).reshape(a.shape)
+        skip_out = _round_fp(out + s, kind).reshape(shape)
+    return out.reshape(shape), skip_out

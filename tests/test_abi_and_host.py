@@ -125,3 +125,10 @@ def test_torch_ops_are_registered_with_meta_implementations():
     assert ops.attention_i8(m((2, 4, 128)), m((2, 16, 128)), m((2, 128, 16)), 1e-3, 0.05, 0.01, 4).shape == (2, 4, 128)
     q8, sc = ops.quantize_per_token_absmax(m((3, 5, 16), torch.float16))
     assert q8.shape == (3, 5, 16) and sc.shape == (3, 5, 1) and sc.dtype == torch.float16
+    y = ops.layer_norm_fwd_fused_single_pass(m((4, 8), torch.bfloat16), m(8, torch.bfloat16), None, 1e-5)
+    assert y.shape == (4, 8) and y.dtype == torch.bfloat16
+    y = ops.skip_layer_norm_fwd_fused_single_pass(m((4, 8), torch.float16), m((4, 8), torch.float16), m(8, torch.float16), None, 1e-5)
+    assert y.shape == (4, 8) and y.dtype == torch.float16
+    o, so = ops.skip_layer_norm_fwd_fused_single_pass2(m((4, 8), torch.float32), m((4, 8), torch.float32), m(8, torch.float32),
+                                                       m(8, torch.float32), 1e-5, True)
+    assert o.shape == so.shape == (4, 8) and so.dtype == torch.float32

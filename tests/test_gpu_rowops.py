@@ -296,3 +296,75 @@ def test_kv_append_i8(S, heads, D, T):
     want_k[:, T - S:, :] = wide[:, 1:H + 1].reshape(S, heads, D).transpose(1, 0, 2)
     want_vt[:, :, T - S:] = wide[:, H + 1:].reshape(S, heads, D).transpose(1, 2, 0)
     assert np.array_equal(cpu(gk), want_k) and np.array_equal(cpu(gv), want_vt)
+
+
+_FP_KINDS = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
+
+
+@pytest.mark.parametrize("rows,cols", [(128, 5120), (33, 768), (7, 4096), (5, 8192), (3, 20480), (9, 1023), (4, 7),
+                                       (2, 1), (16, 2052), (1, 128)])
+@pytest.mark.parametrize("kind", ["f32", "f16", "bf16"])
+def test_layer_norm_fp_and_skip_variants(rows, cols, kind):
+    """layer_norm_fwd_fused_single_pass and the two skip variants against the oracle: fp32 outputs
+    within rtol 1e-5 (+ 1e-5 absolute for values near zero), fp16 / bf16 outputs at most one step
+    of the type apart (the fp32 statistics are summed in another order, which moves a value across a
+    rounding boundary now and then; rate bounded).  The skip output is exact given the LayerNorm output."""
+    fused = _fused()
+    tdt = _FP_KINDS[kind]
+    g = torch.Generator().manual_seed(rows * 31 + cols)
+    x = (torch.randn((rows, cols), generator=g) * 1.3 + 0.2).to(tdt)
+    sk = torch.randn((rows, cols), generator=g).to(tdt)
+    w = (torch.randn(cols, generator=g) * 0.1 + 1.0).to(tdt)
+    b = (torch.randn(cols, generator=g) * 0.1).to(tdt)
+    eps = 1e-5
+    eps_eff = max(eps, 1.6e-5) if kind == "f16" else eps  # kernels/fused.py:502-503
+    xn, skn, wn, bn = (t.float().numpy() for t in (x, sk, w, b))
+    gx, gsk, gw, gb = (t.to(DEV) for t in (x, sk, w, b))
+    ulp = {"f32": 2.0 ** -23, "f16": 2.0 ** -10, "bf16": 2.0 ** -7}[kind]
+
+    def check(got, want):
+        assert got.dtype == tdt and tuple(got.shape) == want.shape
+        got = got.float().cpu().numpy()
+        if kind == "f32":
+            assert np.allclose(got, want, rtol=1e-5, atol=1e-5)
+        else:
+            err = np.abs(got - want)
+            assert np.all(err <= 1.01 * ulp * np.maximum(np.abs(want), 2.0 ** -14)), err.max()
+            assert (err > 0).mean() < 5e-3
+        return got
+
+    for rms in (False, True):
+        for bias in (gb, None):
+            want, _ = O.layer_norm_fp(xn, wn, None if bias is None else bn, eps_eff, rms=rms, kind=kind)
+            out = check(fused.layer_norm_fwd_fused_single_pass(gx, gw, bias, eps, rms), want)
+            o2, s2 = fused.skip_layer_norm_fwd_fused_single_pass2(gx, gsk, gw, bias, eps, rms)
+            assert np.array_equal(o2.float().cpu().numpy(), out)
+            # the skip output: exact given this LayerNorm output
+            want_skip = O._round_fp(out + skn, kind)
+            assert np.array_equal(s2.float().cpu().numpy(), want_skip)
+            s1 = fused.skip_layer_norm_fwd_fused_single_pass(gx, gsk, gw, bias, eps, rms)
+            assert torch.equal(s1, s2)
+    assert torch.equal(gx.cpu(), x) and torch.equal(gsk.cpu(), sk)
+
+
+def test_layer_norm_fp_views_and_errors():
+    fused = _fused()
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn((2, 9, 256), generator=g)
+    w, b = torch.randn(256, generator=g), torch.randn(256, generator=g)
+    want, _ = O.layer_norm_fp(x.numpy(), w.numpy(), b.numpy(), 1e-5)
+    got = fused.layer_norm_fwd_fused_single_pass(x.to(DEV), w.to(DEV), b.to(DEV), 1e-5)
+    assert tuple(got.shape) == (2, 9, 256) and np.allclose(got.cpu().numpy(), want, rtol=1e-5, atol=1e-5)
+    # rows of a wider matrix (row stride 512 elements) and an unaligned column window
+    wide = torch.randn((18, 512), generator=g).to(DEV)
+    for sl in (slice(0, 256), slice(3, 259)):
+        v = wide[:, sl]
+        want, _ = O.layer_norm_fp(v.cpu().numpy(), w.numpy(), b.numpy(), 1e-5)
+        assert np.allclose(fused.layer_norm_fwd_fused_single_pass(v, w.to(DEV), b.to(DEV), 1e-5).cpu().numpy(), want,
+                           rtol=1e-5, atol=1e-5)
+    with pytest.raises(AssertionError):  # dtype mismatch between input and weight (kernels/fused.py:494-496)
+        fused.layer_norm_fwd_fused_single_pass(x.to(DEV).half(), w.to(DEV), b.to(DEV), 1e-5)
+    with pytest.raises(RuntimeError):  # CPU tensors: no fallback
+        fused.layer_norm_fwd_fused_single_pass(x, w, b, 1e-5)
+    empty = fused.layer_norm_fwd_fused_single_pass(torch.empty((0, 256), device=DEV), w.to(DEV), b.to(DEV), 1e-5)
+    assert tuple(empty.shape) == (0, 256)

@@ -184,3 +184,65 @@ def test_quantize_per_token_absmax_vs_the_torch_steps(dtype):
     assert got_s.dtype == want_s.dtype and np.array_equal(got_s, want_s)
     assert np.array_equal(got_q, want_q)
     assert np.abs(got_q[5]).max() == 127 and set(np.unique(got_q[5])) == {127}
+
+
+def test_round_fp_matches_torch_casts():
+    g = torch.Generator().manual_seed(9)
+    v = torch.randn(100000, generator=g) * torch.logspace(-6, 6, 100000)
+    v[:4] = torch.tensor([0.0, -0.0, 1.00390625, 1.01171875])  # bf16 ties: to even both ways
+    assert np.array_equal(O._round_fp(v.numpy(), "bf16"), v.bfloat16().float().numpy())
+    assert np.array_equal(O._round_fp(v.numpy(), "f16"), v.half().float().numpy())
+
+
+@pytest.mark.parametrize("cols", [5, 128, 768, 5120])
+@pytest.mark.parametrize("kind,tdt", [("f32", torch.float32), ("f16", torch.float16), ("bf16", torch.bfloat16)])
+def test_layer_norm_fp_vs_torch_layer_norm(cols, kind, tdt):
+    """The floating-point LayerNorm restatement (kernels/fused.py:385-862) against torch's CPU
+    layer_norm on the same (already rounded) inputs, the skip add against torch's add in the
+    tensors' dtype, RMSNorm against its closed form in float64."""
+    g = torch.Generator().manual_seed(cols)
+    rows = 19
+    x = (torch.randn((rows, cols), generator=g) * 1.7 + 0.3).to(tdt)
+    sk = torch.randn((rows, cols), generator=g).to(tdt)
+    w = (torch.randn(cols, generator=g) * 0.1 + 1.0).to(tdt)
+    b = (torch.randn(cols, generator=g) * 0.1).to(tdt)
+    eps = 1e-5
+    xn, skn, wn, bn = (t.float().numpy() for t in (x, sk, w, b))
+    out, skip_out = O.layer_norm_fp(xn, wn, bn, eps, skip=skn, kind=kind)
+    ref32 = F.layer_norm(x.float(), (cols,), w.float(), b.float(), eps)
+    want = ref32.to(tdt).float().numpy()
+    ulp = {"f32": 2.0 ** -23, "f16": 2.0 ** -10, "bf16": 2.0 ** -7}[kind]
+    # a different summation order moves the fp32 result by a few fp32 ulps: at most one step of the
+    # output type, and only where the value sat on a rounding boundary
+    err = np.abs(out - want)
+    step = ulp * np.maximum(np.abs(want), 2.0 ** -14)
+    assert np.all(err <= (8 if kind == "f32" else 1) * step + (1e-6 if kind == "f32" else 0))
+    if kind != "f32":
+        assert (err > 0).mean() < 5e-3
+    # skip add: exact given `out`
+    want_skip = (torch.from_numpy(out).to(tdt) + sk).float().numpy()
+    assert np.array_equal(skip_out, want_skip)
+    # no bias
+    out_nb, none = O.layer_norm_fp(xn, wn, None, eps, kind=kind)
+    assert none is None
+    ref_nb = F.layer_norm(x.float(), (cols,), w.float(), None, eps).to(tdt).float().numpy()
+    assert np.all(np.abs(out_nb - ref_nb) <= (8 if kind == "f32" else 1) * ulp * np.maximum(np.abs(ref_nb), 2.0 ** -14) + 1e-6)
+    # RMSNorm closed form
+    out_r, _ = O.layer_norm_fp(xn, wn, bn, eps, rms=True, kind=kind)
+    x64 = xn.astype(np.float64)
+    r64 = x64 / np.sqrt((x64 * x64).mean(axis=1, keepdims=True) + eps) * wn + bn
+    assert np.all(np.abs(out_r - r64) <= 2 * ulp * np.maximum(np.abs(r64), 2.0 ** -14) + 1e-6)
+
+
+def test_layer_norm_fp_invariants():
+    """Constant rows hit the eps path (output = bias), a shifted row normalises to the same values."""
+    x = np.full((3, 64), 2.5, np.float32)
+    w = np.linspace(0.5, 1.5, 64).astype(np.float32)
+    b = np.linspace(-1, 1, 64).astype(np.float32)
+    out, _ = O.layer_norm_fp(x, w, b, 1e-5)
+    assert np.array_equal(out, np.broadcast_to(b, out.shape))
+    g = rng(3)
+    y = g.standard_normal((4, 256)).astype(np.float32)
+    o1, _ = O.layer_norm_fp(y, w.repeat(4), None, 1e-5)
+    o2, _ = O.layer_norm_fp(y + np.float32(8.0), w.repeat(4), None, 1e-5)
+    assert np.allclose(o1, o2, rtol=0, atol=2e-5)

@@ -19,7 +19,7 @@ OBJ_DIR = os.path.join(HERE, "_obj")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libtriton_int_hip.so")
 
-SOURCES = ["lib.hip", "gemm_i8.hip", "rowops.hip", "attention_i8.hip", "quant.hip"]
+SOURCES = ["lib.hip", "gemm_i8.hip", "rowops.hip", "attention_i8.hip", "quant.hip", "layernorm_fp.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

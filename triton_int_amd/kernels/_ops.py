@@ -81,6 +81,18 @@ _OPS = {
         "(Tensor x, Tensor weight, Tensor? bias, float eps) -> Tensor",
         lambda x, w, b, eps: _fused.layer_norm_fwd_fused_single_pass_q(x, w, b, eps),
         lambda x, w, b, eps: x.new_empty(x.shape, dtype=torch.int8)),
+    "layer_norm_fwd_fused_single_pass": (
+        "(Tensor x, Tensor weight, Tensor? bias, float eps, bool use_rms_norm=False) -> Tensor",
+        lambda x, w, b, eps, rms=False: _fused.layer_norm_fwd_fused_single_pass(x, w, b, eps, rms),
+        lambda x, w, b, eps, rms=False: x.new_empty(x.shape)),
+    "skip_layer_norm_fwd_fused_single_pass": (
+        "(Tensor x, Tensor skip, Tensor weight, Tensor? bias, float eps, bool use_rms_norm=False) -> Tensor",
+        lambda x, sk, w, b, eps, rms=False: _fused.skip_layer_norm_fwd_fused_single_pass(x, sk, w, b, eps, rms),
+        lambda x, sk, w, b, eps, rms=False: x.new_empty(x.shape)),
+    "skip_layer_norm_fwd_fused_single_pass2": (
+        "(Tensor x, Tensor skip, Tensor weight, Tensor? bias, float eps, bool use_rms_norm=False) -> (Tensor, Tensor)",
+        lambda x, sk, w, b, eps, rms=False: tuple(_fused.skip_layer_norm_fwd_fused_single_pass2(x, sk, w, b, eps, rms)),
+        lambda x, sk, w, b, eps, rms=False: (x.new_empty(x.shape), x.new_empty(x.shape))),
     "dq_add_layernorm_q": (
         "(Tensor input_int32, float input_scale_fp, Tensor residual_input_fp, Tensor gamma, Tensor beta, float eps)"
         " -> (Tensor, Tensor)",

@@ -1,5 +1,5 @@
-"""Fused launchers — the int8 entries of triton_int/kernels/fused.py plus the two ops that file
-only sketches: the dequant + residual-add + LayerNorm + quantise kernel (its Triton stub at
+"""Fused launchers — the entries of triton_int/kernels/fused.py (the int8 ones and the
+floating-point LayerNorm / skip-LayerNorm trio) plus the two ops that file only sketches: the dequant + residual-add + LayerNorm + quantise kernel (its Triton stub at
 kernels/fused.py:17-61 is never launched) and a launchable stand-alone GELU-quant
 (fast_geluQ, kernels/fused.py:76-79, is a device function there).
 """
@@ -50,6 +50,58 @@ def layer_norm_fwd_fused_single_pass_q(x, weight, bias, eps, use_rms_norm=False,
                                     L.ptr(mean), L.ptr(rstd), L.current_stream(x.device))
     L.check(rc, "ti_layernorm_q")
     return (out, mean, rstd) if _return_stats else out
+
+
+def _layernorm_fp(x, skip, weight, bias, eps, use_rms_norm, want_out, want_skip_out):
+    assert x.dtype == weight.dtype, f"input and weight bias must have the same dtype: {x.dtype}, {weight.dtype}"
+    if bias is not None:
+        assert x.dtype == bias.dtype, f"input and bias must have the same dtype: {x.dtype}, {bias.dtype}"
+    assert x.dtype in (torch.float32, torch.float16, torch.bfloat16), f"floating-point LayerNorm takes fp32 / fp16 / bf16, got {x.dtype}"
+    L.require_cuda(x, weight, bias, skip)
+    # catch eps being too small if the tensors are fp16 (kernels/fused.py:501-503)
+    if x.dtype == torch.float16:
+        eps = max(eps, 1.6e-5)
+    N = x.shape[-1]
+    assert weight.numel() == N and (bias is None or bias.numel() == N)
+    a_arg = x.view(-1, N)
+    if a_arg.stride(1) != 1:
+        a_arg = a_arg.contiguous()
+    M = a_arg.shape[0]
+    b_arg = None
+    if skip is not None:
+        assert skip.dtype == x.dtype and skip.numel() == x.numel(), "skip must match the input"
+        b_arg = skip.view(-1, skip.shape[-1])
+        assert tuple(b_arg.shape) == (M, N), "skip must match the input"
+        if b_arg.stride(1) != 1:
+            b_arg = b_arg.contiguous()
+    out = torch.empty(x.shape, dtype=x.dtype, device=x.device) if want_out else None
+    skip_out = torch.empty(x.shape, dtype=x.dtype, device=x.device) if want_skip_out else None
+    weight = weight.contiguous()
+    bias = None if bias is None else bias.contiguous()
+    with L.on_device(x.device):
+        rc = L.lib().ti_layernorm_fp(L.ptr(a_arg), a_arg.stride(0) if M > 1 else N,
+                                     L.ptr(b_arg), (b_arg.stride(0) if M > 1 else N) if b_arg is not None else 0,
+                                     L.TORCH_TO_DT[x.dtype], L.ptr(weight), L.ptr(bias), float(eps),
+                                     int(bool(use_rms_norm)), L.ptr(out), N, L.ptr(skip_out), N, M, N,
+                                     L.current_stream(x.device))
+    L.check(rc, "ti_layernorm_fp")
+    return out, skip_out
+
+
+def layer_norm_fwd_fused_single_pass(x, weight, bias, eps, use_rms_norm=False):
+    """LayerNorm (or RMSNorm) over the last dim, output in x's dtype (fp32 / fp16 / bf16)
+    (reference: kernels/fused.py:486-532)."""
+    return _layernorm_fp(x, None, weight, bias, eps, use_rms_norm, True, False)[0]
+
+
+def skip_layer_norm_fwd_fused_single_pass(x, skip, weight, bias, eps, use_rms_norm=False):
+    """LayerNorm(x) rounded to x's dtype, plus skip (reference: kernels/fused.py:644-693)."""
+    return _layernorm_fp(x, skip, weight, bias, eps, use_rms_norm, False, True)[1]
+
+
+def skip_layer_norm_fwd_fused_single_pass2(x, skip, weight, bias, eps, use_rms_norm=False):
+    """(LayerNorm(x), LayerNorm(x) + skip), both in x's dtype (reference: kernels/fused.py:811-862)."""
+    return _layernorm_fp(x, skip, weight, bias, eps, use_rms_norm, True, True)
 
 
 def dq_add_layernorm_q(input_int32, input_scale_fp, residual_input_fp, gamma, beta, eps, *, quantize=True,
