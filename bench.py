@@ -298,6 +298,20 @@ def extras(torch, dev):
     graph_ms = time_region(torch, graph.replay, 20, 3) / 20
     out["single_linear_512x768x768"] = {"eager_us": eager_ms * 1e3, "graph_us": graph_ms * 1e3,
                                         "TOPS_graph": 2.0 * 512 * 768 * 768 / (graph_ms * 1e-3) / 1e12}
+    del x1, w1, b1, o1
+    # a yardstick, not part of the path: the vendor library's int8 GEMM (torch._int_mm, int32 out) on
+    # the fc1 shape with the same kind of operands, next to this library's int32-output linear
+    try:
+        M, N, K = 2048, 20480, 5120
+        xa = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=dev)
+        wa = torch.randint(-127, 128, (N, K), dtype=torch.int8, device=dev)
+        ba = torch.zeros(N, dtype=torch.int32, device=dev)
+        ours = time_region(torch, lambda: linear.linear_a8_w8_b32_o32(xa, wa, ba), 20, 3)
+        theirs = time_region(torch, lambda: torch._int_mm(xa, wa.t()), 20, 3)
+        out["int32_out_gemm_2048x20480x5120"] = {"this_library_TOPS": 2.0 * M * N * K / ours / 1e9,
+                                                 "torch_int_mm_TOPS": 2.0 * M * N * K / theirs / 1e9}
+    except Exception as ex:  # torch._int_mm is a private API: absent or different elsewhere
+        out["int32_out_gemm_2048x20480x5120"] = {"error": repr(ex)[:120]}
     return out
 
 
