@@ -403,3 +403,37 @@ def test_decode_attention_bmms():
     out = bmm.bmm_s8t_s8n_f32t(gpu(pr), gpu(vt), 1.0 / 16129)
     assert np.array_equal(cpu(out), O.bmm_s8t_s8n_f32t(pr, vt, np.float32(1.0 / 16129)))
     assert np.array_equal(cpu(bmm.bmm_s8t_s8n_s32t(gpu(pr), gpu(vt))), O.bmm_s8t_s8n_s32t(pr, vt))
+
+
+@pytest.mark.parametrize("kind,M,N", [("f32", 32768, 16400), ("i8", 65536, 32784)])
+def test_outputs_beyond_2_gib(kind, M, N):
+    """An output of more than 2^31 bytes: the persistent kernels index it with 32-bit offsets and must
+    not be chosen; whatever runs has to address every row correctly.  K is tiny to keep it cheap;
+    first, last and random rows are checked against numpy's exact integer product."""
+    linear, _, _ = _kl()
+    K = 16
+    g = rng(M + N)
+    a, w = rand_i8(g, M, K), rand_i8(g, N, K)
+    ga, gw = gpu(a), gpu(w)
+    rows = np.concatenate([np.arange(8), np.arange(M - 8, M), g.integers(0, M, size=16),
+                           [2**31 // (N * (4 if kind == "f32" else 1)) + d for d in (-1, 0, 1)]])
+    acc = a[rows].astype(np.int32) @ w.astype(np.int32).T
+    if kind == "f32":
+        bias = g.standard_normal(N).astype(np.float32)
+        out = linear.linear_a8_w8_bfp32_ofp32(ga, gw, gpu(bias), 0.01, 1.0)
+        want = (np.float32(0.01) * acc.astype(np.float32)) + bias * np.float32(1.0)
+        assert out.numel() * 4 > 2**31 and out.dtype == torch.float32
+        got = out[torch.from_numpy(rows).to(DEV)].cpu().numpy()
+        assert np.allclose(got, want, rtol=1e-6, atol=1e-6)
+    else:
+        bias = rand_i8(g, N)
+        out = linear.linear_a8_w8_b8_o8(ga, gw, gpu(bias), 0.002, 0.5)
+        want = O.bmm_i8(a[rows][None], w[None], epilogue=O.EPI_SCALE_I8, out_dtype=O.DT_I8, bias=bias,
+                        alpha=np.float32(0.002), beta=np.float32(0.5))[0]
+        assert out.numel() > 2**31 and out.dtype == torch.int8
+        got = out[torch.from_numpy(rows).to(DEV)].cpu().numpy()
+        assert np.array_equal(got, want)
+    name = _lib().lib().ti_gemm_config_name(_lib().lib().ti_gemm_last_config()).decode()
+    assert not name.startswith(("stream", "ws_")), name
+    del out
+    torch.cuda.empty_cache()
