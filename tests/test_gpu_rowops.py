@@ -368,3 +368,40 @@ def test_layer_norm_fp_views_and_errors():
         fused.layer_norm_fwd_fused_single_pass(x, w, b, 1e-5)
     empty = fused.layer_norm_fwd_fused_single_pass(torch.empty((0, 256), device=DEV), w.to(DEV), b.to(DEV), 1e-5)
     assert tuple(empty.shape) == (0, 256)
+
+
+def test_row_kernels_beyond_2_31_elements():
+    """More than 2^31 elements per tensor: element offsets must be 64-bit.  Inputs are generated on
+    the device; the head, the 2^31 boundary and the tail are checked against the oracle."""
+    fused = _fused()
+    n = 2**31 + 4096 + 3
+    x = torch.empty(n, dtype=torch.float32, device=DEV)
+    gen = torch.Generator(device=DEV).manual_seed(11)
+    for s in range(0, n, 2**28):
+        x[s:s + 2**28].normal_(0.0, 2.0, generator=gen)
+    y = fused.gelu_q(x, 20.0)
+    assert y.numel() == n
+    for lo, hi in ((0, 4096), (2**31 - 2048, 2**31 + 2048), (n - 4099, n)):
+        want = O.gelu_q(x[lo:hi].cpu().numpy(), 20.0)
+        mx, rate = mismatch_report(y[lo:hi].cpu().numpy(), want)
+        assert mx <= 1 and rate < 2e-3, (lo, mx, rate)
+    del y
+    cols = 8192
+    rows = n // cols  # 262144 full rows
+    rows_x = x[:rows * cols].view(rows, cols)
+    g = rng(8)
+    w = (g.normal(1.0, 0.1, cols) / 0.05).astype(np.float32)
+    b = (g.normal(0.0, 0.1, cols) / 0.05).astype(np.float32)
+    # a row stride of cols + 4 elements puts the last rows' offsets beyond 2^31 elements
+    wide = torch.empty((rows, cols + 4), dtype=torch.float32, device=DEV)
+    wide[:, :cols] = rows_x
+    del x, rows_x
+    xs = wide[:, :cols]
+    assert (rows - 1) * (cols + 4) > 2**31
+    q = fused.layer_norm_fwd_fused_single_pass_q(xs, gpu(w), gpu(b), 1e-5)
+    for lo, hi in ((0, 4), (rows - 4, rows), (rows // 2, rows // 2 + 2)):
+        want = O.layernorm_q(xs[lo:hi].cpu().numpy(), w, b, 1e-5)
+        mx, rate = mismatch_report(q[lo:hi].cpu().numpy(), want)
+        assert mx <= 1 and rate < 2e-3, (lo, mx, rate)
+    del wide, q
+    torch.cuda.empty_cache()
