@@ -276,7 +276,11 @@ def extras(torch, dev):
     for name, q_len in (("full", 0), ("causal", S)):
         ms = time_region(torch, lambda: fused.attention_i8(q, k, vt, 1e-3, 0.05, 1.0 / 127.0, causal_q_len=q_len, out=ctx), 10, 2)
         out[f"attention_i8_fused_{name}_160x2048x2048x128"] = {"ms": ms, "scores_per_us": B * S * S / (2 if q_len else 1) / ms / 1e3}
-    del q, k, vt, ctx
+    # decode-sized block: 16 query rows per head against 2048 keys (one pass, one to four workgroups per head)
+    qd, ctxd = q[:40, :16].contiguous(), torch.empty((40, 16, D), dtype=torch.int8, device=dev)
+    ms = time_region(torch, lambda: fused.attention_i8(qd, k[:40], vt[:40], 1e-3, 0.05, 1.0 / 127.0, causal_q_len=16, out=ctxd), 50, 5)
+    out["attention_i8_decode_40x16x2048x128"] = {"ms": ms, "GBps": 2 * 40 * S * D / ms / 1e6}
+    del q, k, vt, ctx, qd, ctxd
     # config 1: one W8A8B8O8Linear 512 x 768 x 768 (launch-latency sized: no roofline claim).  Eager
     # time includes the Python launch path; the graph replay is the kernel alone.
     from triton_int_amd.kernels import linear

@@ -246,6 +246,8 @@ int ti_kv_append_i8(const int8_t* k_src, int64_t k_src_row_stride, const int8_t*
  * (the row's exponentials are summed in a different order).  All columns of a row that share an
  * int8 score flip together, so such a row (about 1 in 10^5 at 2048 keys) can differ from the
  * three-launch result in several output values by a few steps; every other row is identical.
+ * With S <= 16 and T <= 4096 (decode) a one-pass kernel runs instead, one to four workgroups per
+ * batch entry; it takes the exponent against the row maximum like ti_softmax_q.
  * The reference has no fused form (its modules stop at the BMMs, nn/bmm.py:10-74); the
  * three-launch chain remains available and is what this is tested against.
  */

@@ -82,12 +82,14 @@ def test_decoder_layer_prefill_and_decode_small():
     k_old, vt_old = k_cache.clone(), vt_cache.clone()
     hidden_d = g.standard_normal((B, Sd, H), dtype=np.float32)
     tr = {}
+    layer.fused_attention = False  # the three-launch chain first: its stages are checked one by one
     out = layer(gpu(hidden_d), kv_cache=(k_cache, vt_cache), _trace=tr)
     assert out.shape == (B, Sd, H)
     assert torch.equal(k_cache[:, :T - Sd], k_old[:, :T - Sd]) and torch.equal(vt_cache[:, :, :T - Sd], vt_old[:, :, :T - Sd])
     _check_stages(layer, tr, hidden_d, B, Sd, causal_q_len=Sd)
-    # the same decode step through the one-kernel attention (cache offset T - S in the causal mask)
-    layer.fused_attention_min_queries = 1
+    # the same decode step through the one-kernel attention, the default for 16 or fewer query rows
+    # (cache offset T - S in the causal mask)
+    layer.fused_attention = True
     k2, v2 = k_old.clone(), vt_old.clone()
     trf = {}
     layer(gpu(hidden_d), kv_cache=(k2, v2), _trace=trf)
@@ -137,11 +139,21 @@ def test_decoder_layer_opt13b_shapes_run():
     vt_cache = torch.randint(-127, 128, (40, 128, 2048), dtype=torch.int8, generator=g).to(DEV)
     hd = torch.randn((1, 16, 5120), generator=g)
     tr = {}
-    out = layer(hd.to(DEV), kv_cache=(k_cache, vt_cache), _trace=tr)
+    kc2, vc2 = k_cache.clone(), vt_cache.clone()
+    out = layer(hd.to(DEV), kv_cache=(k_cache, vt_cache), _trace=tr)  # layer.fused_attention is off here: the chain
     assert out.shape == (1, 16, 5120) and torch.isfinite(out).all()
     assert np.array_equal(cpu(tr["scores"]), O.bmm_s8t_s8n_s8t(cpu(tr["q"]), cpu(tr["k_all"]), np.float32(layer.qk_alpha)))
     acc = O.linear_a8_w8_b32_o32(cpu(tr["ctx"])[0], cpu(layer.out_proj.weight), cpu(layer.out_proj.bias))
     assert np.array_equal(cpu(tr["acc"])[0], acc)
+    # the default decode path (one attention kernel per step): same context, same layer output
+    layer.fused_attention = True
+    trf = {}
+    out_f = layer(hd.to(DEV), kv_cache=(kc2, vc2), _trace=trf)
+    assert trf["scores"] is None and torch.equal(kc2, k_cache) and torch.equal(vc2, vt_cache)
+    bad_rows = int(((trf["ctx"].int() - tr["ctx"].int()).abs().view(16, 40, 128).amax(dim=-1) > 0).sum())
+    assert bad_rows <= 1
+    if bad_rows == 0:
+        assert torch.equal(out_f, out)
 
 
 def test_layer_replayed_from_a_hip_graph_matches_eager():

@@ -222,6 +222,30 @@ def test_attention_i8_against_the_three_kernel_chain(BH, S, T, q_len):
     assert seen_nontrivial or T >= 1024  # long rows of random scores spread the probabilities below 1/254
 
 
+@pytest.mark.parametrize("BH,S,T,q_len", [(40, 16, 2048, 16), (3, 5, 80, 5), (2, 16, 4096, 0), (2, 9, 1040, 9),
+                                           (5, 16, 1024, 16), (2, 7, 3008, 7), (1, 16, 16, 16), (3, 2, 2064, 0),
+                                           (2, 12, 48, 4)])
+def test_attention_i8_few_query_rows(BH, S, T, q_len):
+    """16 or fewer query rows per head (decode, short chunks) run the one-workgroup-per-head kernel:
+    same checker and same bar as above.  Its exponent is taken against the row maximum like the
+    stand-alone softmax kernel's, so only the order of a row's sum differs from the chain."""
+    fused = _fused()
+    g = rng(BH * 77 + S * 5 + T)
+    D = 128
+    q = g.integers(-127, 128, size=(BH, S, D), dtype=np.int8)
+    k = g.integers(-127, 128, size=(BH, T, D), dtype=np.int8)
+    vt = g.integers(-127, 128, size=(BH, D, T), dtype=np.int8)
+    for qk_alpha, score_scale, pv_alpha in ((1e-3, 0.05, 1.0 / 127.0), (4e-3, 0.02, 0.03), (2e-3, 0.3, 0.02)):
+        want = O.attention_i8(q, k, vt, qk_alpha, score_scale, pv_alpha, causal_q_len=q_len)
+        out = torch.full((BH, S, D), 77, dtype=torch.int8, device=DEV)
+        fused.attention_i8(gpu(q), gpu(k), gpu(vt), qk_alpha, score_scale, pv_alpha, causal_q_len=q_len, out=out)
+        got = cpu(out)
+        mx, rate = mismatch_report(got, want)
+        bad_rows = int((np.abs(got.astype(int) - want.astype(int)).max(axis=-1) > 0).sum())
+        print(f"attention_i8 (few rows) BH {BH} S {S} T {T} q_len {q_len} scale {score_scale}: max diff {mx}, rows {bad_rows}")
+        assert bad_rows <= max(1, BH * S // 200), f"{bad_rows} rows differ (max {mx})"
+
+
 def test_attention_i8_strided_views_and_errors():
     fused = _fused()
     g = rng(77)

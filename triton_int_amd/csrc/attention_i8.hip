@@ -21,6 +21,8 @@
 // from the accumulator registers (two half-wave swaps put a row's keys in order) and feeds them
 // to the P.V MFMAs, so P never goes through memory.
 //
+// (Blocks of 16 or fewer query rows take attention_decode_i8_kernel further down instead.)
+//
 // Workgroup = 4 waves = 128 query rows of one head; a wave owns 32 rows.  K and V^T are staged
 // through LDS in tiles of 64 keys, double-buffered, one barrier per tile.  Causal masking skips
 // whole key tiles beyond a wave's last visible key and masks inside the tiles on the diagonal.
@@ -284,6 +286,178 @@ __global__ __launch_bounds__(256, 2) void attention_i8_kernel(AttnParams p) {
   }
 }
 
+
+// ---- few query rows (decode): one workgroup per head ------------------------------------------------
+//
+// With 16 or fewer query rows per head a head's whole attention fits one workgroup: 16 waves, one
+// pass.  Wave w computes the scores of the 16-key chunks w, w + 16, ... with 16x16x64 MFMAs (K rows
+// loaded from memory straight into the operand layout: 16 rows x 64 bytes per instruction) and keeps
+// them in registers; row maximum and sum go through LDS; the int8 probabilities are written to LDS in
+// key order ([16 queries][T]), from where every wave reads them back as MFMA operands for P.V: wave w
+// owns 16 of the 128 output columns (V^T rows, also loaded straight into the operand layout) and
+// one half of the 64-key groups; the two halves meet in LDS.  The arithmetic is that of the three
+// kernels (score quantisation, exponent against the row maximum, 127 / sum, context quantisation);
+// only the order of a row's sum differs.
+constexpr int AD_WAVES = 16;
+constexpr int AD_MAXT = 4096;
+
+// CPW: 16-key chunks per wave (T <= 256 * CPW).  DBW: 16-column blocks of the output a workgroup
+// produces (8: the whole head; fewer: the head is spread over 8 / DBW workgroups, each of which
+// repeats the scores and the softmax and reads only its rows of V^T — a single CU fills its caches at
+// about 30 GB/s, so a head's 512 KB of K and V^T through one CU alone would take 17 us).
+template <int CPW, int DBW>
+__global__ __launch_bounds__(AD_WAVES * 64) void attention_decode_i8_kernel(AttnParams p) {
+  constexpr int TMAX = 256 * CPW;
+  constexpr int PP = TMAX + 16;             // LDS pitch of a query's probabilities
+  constexpr int KPARTS = AD_WAVES / DBW;    // waves that share an output block and split the keys
+  constexpr int GPW = (TMAX / 64 + KPARTS - 1) / KPARTS;  // 64-key groups per wave in P.V
+  constexpr int HOIST = CPW >= 16 ? (GPW < 4 ? GPW : 4) : GPW;  // V^T operands fetched before the softmax reductions
+  __shared__ __attribute__((aligned(16))) char p_lds[16 * PP];
+  __shared__ float red_max[AD_WAVES][16];
+  __shared__ float red_sum[AD_WAVES][16];
+  __shared__ __attribute__((aligned(16))) v4i ctx_red[AD_WAVES][64];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n = lane & 15, kq = lane >> 4;  // operand row / 16-byte quarter of a 64-deep k-step
+  // the workgroups of a head are p.batch apart: with a batch that is a multiple of 8 they run on the
+  // same XCD and share its L2 for K
+  const int bh = blockIdx.x % p.batch;
+  const int dbase = (blockIdx.x / p.batch) * DBW;
+  const int OOB = 0x7ffffff0;
+  const float MAGIC = 12582912.0f;
+  const __amdgpu_buffer_rsrc_t rQ =
+      __builtin_amdgcn_make_buffer_rsrc((void*)(p.q + (int64_t)bh * p.sQb), 0, (int)((p.S - 1) * p.sQm + AT_D), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rK =
+      __builtin_amdgcn_make_buffer_rsrc((void*)(p.k + (int64_t)bh * p.sKb), 0, (int)((p.T - 1) * p.sKn + AT_D), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rV =
+      __builtin_amdgcn_make_buffer_rsrc((void*)(p.vt + (int64_t)bh * p.sVb), 0, (int)((AT_D - 1) * p.sVd + p.T), 0x00020000);
+  const int NCH = p.T >> 4;         // 16-key chunks
+  const int NG = (p.T + 63) >> 6;   // 64-key groups
+  const int db = dbase + wave % DBW, kh = wave / DBW;
+
+  // ---- scores: f = int8 score + 128 as a float, -inf where masked or beyond T
+  v4i qf[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks)
+    qf[ks] = __builtin_amdgcn_raw_buffer_load_b128(rQ, n < p.S ? n * (int)p.sQm + ks * 64 + kq * 16 : OOB, 0, 0);
+  const int limit = p.causal_q_len > 0 ? min(p.T, (n % p.causal_q_len) + (p.T - p.causal_q_len) + 1) : p.T;
+  const float NEG = -__builtin_inff();
+  float f[CPW][4];
+  constexpr int NB = CPW < 8 ? CPW : (CPW > 8 ? 4 : 8);  // chunks whose K operands are in flight together
+#pragma unroll
+  for (int b0 = 0; b0 < CPW; b0 += NB) {
+    v4i kf[NB][2];
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      const int c = wave + AD_WAVES * (b0 + i);
+      const int off = (c * 16 + n) * (int)p.sKn + kq * 16;
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) kf[i][ks] = __builtin_amdgcn_raw_buffer_load_b128(rK, c < NCH ? off + ks * 64 : OOB, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      const int c = wave + AD_WAVES * (b0 + i);
+      v4i acc = {0, 0, 0, 0};
+      acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(kf[i][0], qf[0], acc, 0, 0, 0);
+      acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(kf[i][1], qf[1], acc, 0, 0, 0);
+      // acc[r]: key c*16 + 4*kq + r, query n
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float v = (float)acc[r] * p.qk_alpha;
+        v = __builtin_amdgcn_fmed3f(v, -128.0f, 127.0f);
+        const int key = c * 16 + 4 * kq + r;
+        f[b0 + i][r] = key < limit ? __builtin_rintf(v) + 128.0f : NEG;
+      }
+    }
+  }
+  // V^T operands of this wave's first groups: in flight during the reductions below
+  v4i vf[HOIST];
+#pragma unroll
+  for (int i = 0; i < HOIST; ++i) {
+    const int g = kh + KPARTS * i;
+    const int col = 64 * g + 16 * kq;
+    vf[i] = __builtin_amdgcn_raw_buffer_load_b128(rV, col < p.T ? (16 * db + n) * (int)p.sVd + col : OOB, 0, 0);
+  }
+
+  // ---- row maximum (exact: integers), exponentials, row sum
+  float mx = NEG;
+#pragma unroll
+  for (int i = 0; i < CPW; ++i) mx = fmaxf(fmaxf(mx, fmaxf(f[i][0], f[i][1])), fmaxf(f[i][2], f[i][3]));
+  mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  if (kq == 0) red_max[wave][n] = mx;
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < AD_WAVES; ++w) mx = fmaxf(mx, red_max[w][n]);
+  const float c0 = -(mx * p.s2);
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < CPW; ++i)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      f[i][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(f[i][r], p.s2, c0));
+      sum += f[i][r];
+    }
+  sum += __shfl_xor(sum, 16, 64);
+  sum += __shfl_xor(sum, 32, 64);
+  if (kq == 0) red_sum[wave][n] = sum;
+  __syncthreads();
+  sum = 0.0f;
+#pragma unroll
+  for (int w = 0; w < AD_WAVES; ++w) sum += red_sum[w][n];
+  const float rcp = 127.0f / sum;
+
+  // ---- int8 probabilities into LDS, key order; keys in [T, 64 * NG) get zeros (their f is -inf)
+#pragma unroll
+  for (int i = 0; i < CPW; ++i) {
+    const int c = wave + AD_WAVES * i;
+    if (c < 4 * NG) {
+      const unsigned b0 = __float_as_uint(__builtin_fmaf(f[i][0], rcp, MAGIC)), b1 = __float_as_uint(__builtin_fmaf(f[i][1], rcp, MAGIC));
+      const unsigned b2 = __float_as_uint(__builtin_fmaf(f[i][2], rcp, MAGIC)), b3 = __float_as_uint(__builtin_fmaf(f[i][3], rcp, MAGIC));
+      *(unsigned*)(p_lds + n * PP + 16 * c + 4 * kq) =
+          __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u) | __builtin_amdgcn_perm(b3, b2, 0x04000c0cu);
+    }
+  }
+  __syncthreads();
+
+  // ---- P.V: D[d = 16*db + 4*kq + r][query n] over this wave's key groups
+  v4i o = {0, 0, 0, 0};
+#pragma unroll
+  for (int i = 0; i < HOIST; ++i) {
+    const int g = kh + KPARTS * i;
+    if (g < NG) o = __builtin_amdgcn_mfma_i32_16x16x64_i8(vf[i], *(const v4i*)(p_lds + n * PP + 64 * g + 16 * kq), o, 0, 0, 0);
+  }
+#pragma unroll
+  for (int i0 = HOIST; i0 < GPW; i0 += 4) {
+    v4i vb[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int col = 64 * (kh + KPARTS * (i0 + i)) + 16 * kq;
+      vb[i] = __builtin_amdgcn_raw_buffer_load_b128(rV, col < p.T ? (16 * db + n) * (int)p.sVd + col : OOB, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int g = kh + KPARTS * (i0 + i);
+      if (g < NG) o = __builtin_amdgcn_mfma_i32_16x16x64_i8(vb[i], *(const v4i*)(p_lds + n * PP + 64 * g + 16 * kq), o, 0, 0, 0);
+    }
+  }
+  if (kh > 0) ctx_red[wave][lane] = o;
+  __syncthreads();
+  if (kh == 0 && n < p.S) {
+#pragma unroll
+    for (int k2 = 1; k2 < KPARTS; ++k2) o += ctx_red[wave + k2 * DBW][lane];
+    unsigned b[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float v = (float)o[r] * p.pv_alpha;
+      v = __builtin_amdgcn_fmed3f(v, -128.0f, 127.0f);
+      b[r] = __float_as_uint(v + MAGIC);
+    }
+    *(unsigned*)(p.out + (int64_t)bh * p.sOb + (int64_t)n * p.sOm + 16 * db + 4 * kq) =
+        __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u) | __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);
+  }
+}
+
 }  // namespace ti
 
 extern "C" int ti_attention_i8(const int8_t* q, int64_t q_batch_stride, int64_t q_row_stride, const int8_t* k,
@@ -312,6 +486,9 @@ extern "C" int ti_attention_i8(const int8_t* q, int64_t q_batch_stride, int64_t 
   const float s2 = score_scale * 1.44269504088896340736f;
   if (!(score_scale > 0.0f) || s2 * 255.0f > 120.0f)
     return fail(TI_E_COMBO, "score_scale %g outside (0, 0.32]: use the three-kernel path", (double)score_scale);
+  const int64_t lim32 = (int64_t)1 << 31;
+  const bool few_rows = S <= 16 && T <= AD_MAXT && (int64_t)T * k_row_stride < lim32 && (int64_t)AT_D * vt_row_stride < lim32 &&
+                        (int64_t)S * q_row_stride < lim32;
   int rc = check_device();
   if (rc != TI_OK) return rc;
   AttnParams p;
@@ -322,6 +499,23 @@ extern "C" int ti_attention_i8(const int8_t* q, int64_t q_batch_stride, int64_t 
   p.qk_alpha = qk_alpha; p.s2 = s2; p.pv_alpha = pv_alpha;
   p.nblk = (S + AT_ROWS - 1) / AT_ROWS;
   p.batch = batch;
+  if (few_rows) {
+    // spread a head over as many workgroups as keep the launch within one round of the 256 CUs
+    // (measured, 40 heads x 16 rows x 2048 keys: 18.9 / 15.3 / 13.6 us for 1 / 2 / 4 workgroups per head,
+    // 24 us for 8, which no longer fit one round)
+    int dbw = 8;
+    while (dbw > 1 && (int64_t)batch * (16 / dbw) <= 256) dbw /= 2;
+    const dim3 grid((unsigned)(batch * (8 / dbw))), block(AD_WAVES * 64);
+    const hipStream_t st = (hipStream_t)stream;
+#define TI_AD_LAUNCH(C) \
+    (dbw == 8 ? attention_decode_i8_kernel<C, 8><<<grid, block, 0, st>>>(p) : dbw == 4 ? attention_decode_i8_kernel<C, 4><<<grid, block, 0, st>>>(p) \
+     : dbw == 2 ? attention_decode_i8_kernel<C, 2><<<grid, block, 0, st>>>(p) : attention_decode_i8_kernel<C, 1><<<grid, block, 0, st>>>(p))
+    if (T <= 1024) TI_AD_LAUNCH(4);
+    else if (T <= 2048) TI_AD_LAUNCH(8);
+    else TI_AD_LAUNCH(16);
+#undef TI_AD_LAUNCH
+    return launch_status("attention_decode_i8_kernel");
+  }
   attention_i8_kernel<<<dim3((unsigned)(p.nblk * batch)), dim3(256), 0, (hipStream_t)stream>>>(p);
   return launch_status("attention_i8_kernel");
 }

@@ -11,8 +11,8 @@ end-to-end tests: every heavy step is one of the package's HIP kernels, torch on
       scores = BMM_S8T_S8N_S8T(q, k) -> int8                (bmm_s8t_s8n_s8t)
       probs  = softmax_q(scores, causal) -> int8 [0,127]    (ti_softmax_q)
       ctx    = BMM_S8T_S8N_S8T(probs, v^T) -> int8, written head-merged through output strides
-               (with `fused_attention`, the default for 128 or more query positions, these three run
-               as one kernel, ti_attention_i8, and scores / probabilities never reach memory)
+               (with `fused_attention`, the default for 128 or more query positions and for 16 or fewer,
+               these three run as one kernel, ti_attention_i8, and scores / probabilities never reach memory)
       acc    = W8A8B32O32LinearWithoutScaling(ctx) -> int32 (linear_a8_w8_b32_o32)   out_proj
       resid, h8 = DQ_Add_LayerNorm_Q(hidden, acc)           (ti_dq_add_layernorm_q)
       f8     = W8A8BFP32OFP32_GeLu_Q(h8) -> int8            (GEMM + GELU-quant epilogue)   fc1
@@ -47,8 +47,8 @@ class W8A8OPTDecoderLayer(torch.nn.Module):
         self.qk_alpha = 1e-3
         self.score_scale = 0.05
         self.pv_alpha = 1.0 / 127.0
-        # one-kernel attention for prefill-sized blocks of queries; the three-launch chain otherwise
-        # (a handful of query rows per head leaves that kernel too few workgroups)
+        # one-kernel attention for prefill-sized blocks of queries and for decode-sized ones (16 or fewer
+        # rows per head); the three-launch chain in between (too few workgroups for the block kernel)
         self.fused_attention = True
         self.fused_attention_min_queries = 128
 
@@ -143,8 +143,9 @@ class W8A8OPTDecoderLayer(torch.nn.Module):
         mark("kv_append_v_transpose")
         T = k_all.shape[1]
         ctx = torch.empty((B, S, H), dtype=torch.int8, device=hidden.device)
-        fused = (self.fused_attention and S >= self.fused_attention_min_queries and self.head_dim == 128
-                 and T % 16 == 0 and 0.0 < self.score_scale <= 0.32)
+        # 16 or fewer query rows (decode) against up to 4096 keys run the kernel's one-workgroup-per-head form
+        fused = (self.fused_attention and (S >= self.fused_attention_min_queries or (S <= 16 and T <= 4096))
+                 and self.head_dim == 128 and T % 16 == 0 and 0.0 < self.score_scale <= 0.32)
         scores = probs = None
         if fused:
             for b in range(B):
