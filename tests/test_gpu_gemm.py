@@ -437,3 +437,40 @@ def test_outputs_beyond_2_gib(kind, M, N):
     assert not name.startswith(("stream", "ws_")), name
     del out
     torch.cuda.empty_cache()
+
+
+def test_decode_kernel_several_passes_strided_and_16bit_outputs():
+    """The M <= 16 weight-streaming kernel where a workgroup needs several passes over K (more than
+    32 units of 4 weight rows each: a vocabulary-sized N), with a ragged N, with outputs that are rows
+    of a wider matrix or have a non-unit column stride (element-wise stores), and with fp16 / bf16
+    outputs (4 elements = one 8-byte store)."""
+    linear, _, _ = _kl()
+    L = _lib()
+    g = rng(99)
+    M, N, K = 16, 50272 + 2, 1024
+    a, w = rand_i8(g, M, K, lo=-128), rand_i8(g, N, K, lo=-128)
+    b32 = g.integers(-2**20, 2**20, size=N, dtype=np.int32)
+    b8 = rand_i8(g, N); bf = g.standard_normal(N).astype(np.float32)
+    ga, gw = gpu(a), gpu(w)
+    got = cpu(linear.linear_a8_w8_b32_o32(ga, gw, gpu(b32)))
+    assert L.lib().ti_gemm_config_name(L.lib().ti_gemm_last_config()).decode().startswith("rows4")
+    assert np.array_equal(got, O.linear_a8_w8_b32_o32(a, w, b32))
+    alpha = np.float32(40.0 / (np.sqrt(K) * 127 * 127 / 3)); beta = np.float32(0.05)
+    want8 = O.linear_a8_w8_b8_o8(a, w, b8, alpha, beta)
+    assert np.array_equal(cpu(linear.linear_a8_w8_b8_o8(ga, gw, gpu(b8), alpha, beta)), want8)
+    # rows of a wider matrix, starting at an odd column (unaligned: element-wise stores)
+    wide = torch.zeros((M, N + 7), dtype=torch.int8, device=DEV)
+    linear.linear_a8_w8_b8_o8(ga, gw, gpu(b8), alpha, beta, out=wide[:, 3:3 + N])
+    assert np.array_equal(cpu(wide)[:, 3:3 + N], want8) and not cpu(wide)[:, :3].any() and not cpu(wide)[:, 3 + N:].any()
+    # transposed output (column stride != 1)
+    M2, N2, K2 = 7, 644, 2064
+    a2, w2 = rand_i8(g, M2, K2), rand_i8(g, N2, K2)
+    bf2 = g.standard_normal(N2).astype(np.float32)
+    outT = torch.zeros((N2, M2), dtype=torch.float32, device=DEV)
+    cfg = [i for i, nm in _configs(M2) if nm.startswith("rows4")][0]
+    linear.linear_a8_w8_bfp32_ofp32(gpu(a2), gpu(w2), gpu(bf2), alpha, 1.0, out=outT.t(), _config=cfg)
+    assert np.array_equal(cpu(outT).T, O.linear_a8_w8_bfp32_ofp32(a2, w2, bf2, alpha, 1.0))
+    # 16-bit outputs
+    for dt, odt in ((torch.float16, O.DT_F16), (torch.bfloat16, O.DT_BF16)):
+        got16 = cpu(linear.linear_a8_w8_bfp32_ofp32(ga, gw, gpu(bf), alpha, 1.0, dtype=dt))
+        assert np.array_equal(got16, O.linear_a8_w8_bfp32_ofp32(a, w, bf, alpha, 1.0, out_dtype=odt))

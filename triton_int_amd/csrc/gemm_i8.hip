@@ -154,6 +154,22 @@ __device__ __forceinline__ void store_one(const EpiCtx& e, void* C, int64_t off,
   }
 }
 
+// the same conversions, returned as the output element's bits (for callers that pack several
+// elements into one store)
+template <int OUTCLS>
+__device__ __forceinline__ unsigned convert_one(const EpiCtx& e, int acc, float col, int bias_i32, int out_dtype) {
+  if constexpr (OUTCLS == OUT8) {
+    return (unsigned)epi_q8(e, acc, col) & 0xffu;
+  } else if constexpr (OUTCLS == OUT32) {
+    if (e.epilogue == TI_EPI_I32) return (unsigned)acc + (unsigned)bias_i32;
+    if (e.epilogue == TI_EPI_SCALE_I32) return (unsigned)q32(epi_value(e, acc, col), e.round_mode);
+    return __float_as_uint(epi_value(e, acc, col));
+  } else {
+    const float v = epi_value(e, acc, col);
+    return out_dtype == TI_F16 ? f32_to_f16_bits(v) : f32_to_bf16_bits(v);
+  }
+}
+
 __device__ __forceinline__ EpiCtx make_epi(const GemmParams& p, int bz) {
   EpiCtx e;
   const int64_t si = (int64_t)bz * p.scale_bs;
@@ -1430,6 +1446,47 @@ __global__ __launch_bounds__(512, UU ? 2 : 4) void gemm_skinny_kernel(GemmParams
 constexpr int R4_NW = 8, R4_RG = 4, R4_KC = 1024, R4_PITCH = R4_KC + 16, R4_WPITCH = R4_KC + 64, R4_NST = 3, R4_XB = 3,
               R4_UMAX = 4;
 
+// The store phase of gemm_rows4_kernel's epilogue: thread t of the 512 consumer threads takes row t / 32
+// and the 4 outputs of unit unit0 + t % 32 from the LDS tile (row r at tile0 + (r/2) * ring + (r%2) * 2048),
+// converts them and stores them as one piece, so a row's outputs leave as one contiguous run.  A
+// function of its own: inlined, its operands cost the main loop registers.
+template <int OUTCLS>
+__device__ __attribute__((noinline)) void rows4_store_tile(const EpiCtx e, char* Cz, int64_t sCm, int64_t sCn, int M, int N,
+                                                          int out_dtype, unsigned tile0, int tid, int unit0, int u_end,
+                                                          int max_units) {
+  constexpr int ESZ = OUTCLS == OUT8 ? 1 : (OUTCLS == OUT32 ? 4 : 2);
+  constexpr int RING = R4_NST * R4_RG * R4_WPITCH;
+  const int row = tid >> 5, grp = tid & 31;
+  const int unit = unit0 + grp;
+  if (!(row < M && unit < u_end && grp < max_units)) return;
+  const unsigned addr = tile0 + (row >> 1) * RING + (row & 1) * 2048 + grp * 16;
+  const v4i a = *(const __attribute__((address_space(3))) v4i*)(uintptr_t)addr;
+  const int n0 = unit * R4_RG;
+  unsigned b[R4_RG];
+#pragma unroll
+  for (int i = 0; i < R4_RG; ++i) {
+    const int n = min(n0 + i, N - 1);
+    const int bias_i32 = (e.epilogue == TI_EPI_I32 && e.bias_kind == TI_BIAS_I32) ? ((const int*)e.bias)[n] : 0;
+    b[i] = convert_one<OUTCLS>(e, a[i], column_term(e, n), bias_i32, out_dtype);
+  }
+  char* dst = Cz + ((int64_t)row * sCm + (int64_t)n0 * sCn) * ESZ;
+  if (sCn == 1 && n0 + R4_RG <= N && (((uintptr_t)dst) & (R4_RG * ESZ - 1)) == 0) {
+    if constexpr (OUTCLS == OUT8) *(unsigned*)dst = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
+    else if constexpr (OUTCLS == OUT32) *(v4u*)dst = (v4u){b[0], b[1], b[2], b[3]};
+    else *(uint2*)dst = make_uint2(b[0] | (b[1] << 16), b[2] | (b[3] << 16));
+  } else {
+#pragma unroll
+    for (int i = 0; i < R4_RG; ++i) {
+      if (n0 + i < N) {
+        char* d = dst + (int64_t)i * sCn * ESZ;
+        if constexpr (OUTCLS == OUT8) *(int8_t*)d = (int8_t)b[i];
+        else if constexpr (OUTCLS == OUT32) *(unsigned*)d = b[i];
+        else *(uint16_t*)d = (uint16_t)b[i];
+      }
+    }
+  }
+}
+
 template <int OUTCLS>
 __global__ __launch_bounds__((R4_NW + 1) * 64) void gemm_rows4_kernel(GemmParams p) {
   constexpr int STAGE = R4_RG * R4_WPITCH;  // one job: 4 rows x 1 KB (+ padding against bank conflicts)
@@ -1468,12 +1525,18 @@ __global__ __launch_bounds__((R4_NW + 1) * 64) void gemm_rows4_kernel(GemmParams
     };
     issue_x(0);
     issue_x(1);
+    int left = NCH;  // chunks until the end of the pass
     for (int g = 0; g < total; ++g) {
       wait_loads_and_barrier<16>();  // chunk g has landed (chunk g+1 may be in flight); hand it over
       issue_x(g + 2);                // into the buffer of chunk g-1, whose readers passed the barrier
+      if (--left == 0) {
+        // end of a pass: the consumers' reduction barrier (K split) and the two of their epilogue
+        left = NCH;
+        if (KS > 1) asm volatile("s_barrier" ::: "memory");
+        asm volatile("s_barrier\n\ts_barrier" ::: "memory");
+      }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    if (KS > 1) asm volatile("s_barrier" ::: "memory");  // the consumers' reduction barrier
     return;
   }
 
@@ -1550,30 +1613,29 @@ __global__ __launch_bounds__((R4_NW + 1) * 64) void gemm_rows4_kernel(GemmParams
           if (ui < nu) *(v4i*)(ring_p + ui * 1024 + lane * 16) = acc[ui];
       }
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-      if (kpart == 1) return;
-      const char* other = ring_p + NSLOT * (R4_NST * STAGE);
+      if (kpart == 0) {
+        const char* other = ring_p + NSLOT * (R4_NST * STAGE);
 #pragma unroll
-      for (int ui = 0; ui < R4_UMAX; ++ui)
-        if (ui < nu) acc[ui] += *(const v4i*)(other + ui * 1024 + lane * 16);
-    }
-    // acc[ui][i], lanes 0..15: n = unit*4 + i, m = lane
-    if (c4 == 0 && r16 < p.M) {
-#pragma unroll
-      for (int ui = 0; ui < R4_UMAX; ++ui) {
-        if (ui < nu) {
-          const int n0 = (u_first + ui * NSLOT) * R4_RG;
-#pragma unroll
-          for (int i = 0; i < R4_RG; ++i) {
-            const int n = n0 + i;
-            if (n < p.N) {
-              const int bias_i32 = (e.epilogue == TI_EPI_I32 && e.bias_kind == TI_BIAS_I32) ? ((const int*)e.bias)[n] : 0;
-              store_one<OUTCLS>(e, Cz, (int64_t)r16 * p.sCm + (int64_t)n * p.sCn, acc[ui][i], column_term(e, n), bias_i32,
-                                p.out_dtype);
-            }
-          }
-        }
+        for (int ui = 0; ui < R4_UMAX; ++ui)
+          if (ui < nu) acc[ui] += *(const v4i*)(other + ui * 1024 + lane * 16);
       }
     }
+    // ---- epilogue.  acc[ui][i], lanes 0..15: n = unit*4 + i, m = lane.  The workgroup's units of a pass
+    // are consecutive, so its outputs are 16 rows x (4 x units) consecutive columns: the sums go to
+    // an LDS tile (row r in the third ring slot of wave r/2, which no load touches before the next
+    // pass's first chunk barrier) and leave as whole row pieces, 4 elements per thread, instead of
+    // single elements scattered over 16 rows (20480 x 5120: 2.5 us of a 22.5 us launch).  Every load
+    // of every wave has landed before the tile is written (first barrier); the second publishes it.
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    auto tile_row = [&](int r) -> char* { return lds + R4_XB * XBUF + (r >> 1) * (R4_NST * STAGE) + 2 * STAGE + (r & 1) * 2048; };
+    if (kpart == 0 && c4 == 0) {
+#pragma unroll
+      for (int ui = 0; ui < R4_UMAX; ++ui)
+        if (ui < nu) *(v4i*)(tile_row(r16) + (slot + ui * NSLOT) * 16) = acc[ui];
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    rows4_store_tile<OUTCLS>(e, Cz, p.sCm, p.sCn, p.M, p.N, p.out_dtype, lds_base + R4_XB * XBUF + 2 * STAGE, tid,
+                             ub0 + pass * (NSLOT * R4_UMAX), u_end, NSLOT * R4_UMAX);
   }
 }
 
@@ -1802,12 +1864,12 @@ static int run(GemmParams p, int config, hipStream_t stream) {
     // few weight rows: two waves per unit (even / odd chunks of K), so that every wave streams
     const int units = (p.N + R4_RG - 1) / R4_RG;
     p.ksplit = (units <= 1024 && p.K > R4_KC) ? 2 : 1;
-    // every wave of a workgroup gets the same number of units (they meet at a barrier per chunk
-    // of K), and the workgroups fit the chip in one round
-    const int slots = R4_NW / p.ksplit;
-    // fewer units than wave slots on the chip: spread them over all 256 CUs (some waves of a
-    // workgroup then have no unit; they only join the barriers)
-    const int per = units < slots * 256 ? (units + 255) / 256 : slots * ((units + slots * 256 - 1) / (slots * 256));
+    // One workgroup per CU (its LDS allows no second one), all batches together in one round of
+    // the 256 CUs, every CU busy: what a CU can pull from memory is the limit (about 27 GB/s each),
+    // so an idle CU costs more than waves of a workgroup that carry one unit less than others
+    // (three grouped 5120 x 5120 projections: 25.6 -> 17.9 us).
+    const int wgs = p.batch >= 256 ? 1 : 256 / p.batch;
+    const int per = (units + wgs - 1) / wgs;
     const int blocks = (units + per - 1) / per;
     g_last_config = config;
     k.fn[out_class(p.out_dtype)]<<<dim3((unsigned)blocks, (unsigned)p.batch), dim3(k.threads), 0, stream>>>(p);
