@@ -177,3 +177,32 @@ def test_registered_torch_ops_dispatch_and_trace():
 
     compiled = torch.compile(f, backend="eager", fullgraph=True)
     assert torch.equal(compiled(ga), f(ga))
+
+
+def test_dynamic_w8a8_linear_tracks_the_float_module():
+    """The dynamically quantised linear (per-tensor absmax of the activation at every call): the
+    int8 GEMM and its fp32 epilogue are checked against the oracle on the int8 activations the module
+    itself formed from a numpy restatement of the helper, and the result tracks the float module."""
+    from triton_int_amd.nn.linear import DanymicW8A8BFP32OFP32Linear, DynamicW8A8BFP32OFP32Linear
+    assert DanymicW8A8BFP32OFP32Linear is DynamicW8A8BFP32OFP32Linear
+    torch.manual_seed(3)
+    lin = torch.nn.Linear(256, 192)
+    x = torch.randn(3, 17, 256) * 2.5
+    want_float = lin(x).detach()
+    q = DynamicW8A8BFP32OFP32Linear.from_float(_clone_linear(lin)).to(DEV)
+    gx = x.to(DEV)
+    y = q(gx)
+    assert y.shape == (3, 17, 192) and y.dtype == torch.float32 and torch.equal(gx.cpu(), x)  # x untouched
+    xs = x.numpy().reshape(-1, 256)
+    scale = np.float32(np.abs(xs).max()) / np.float32(127)
+    x8 = np.rint(xs / scale).astype(np.int8)
+    alpha = np.float32(scale * np.float32(float(q.weight_scale)))
+    want = O.linear_a8_w8_bfp32_ofp32(x8, cpu(q.weight), cpu(q.bias), alpha, np.float32(1.0))
+    assert np.allclose(cpu(y).reshape(-1, 192), want, rtol=1e-5, atol=1e-6)
+    assert (y.cpu() - want_float).abs().max() < 0.15  # two 8-bit quantisations of a 256-term sum
+
+
+def _clone_linear(lin):
+    c = torch.nn.Linear(lin.in_features, lin.out_features)
+    c.load_state_dict(lin.state_dict())
+    return c

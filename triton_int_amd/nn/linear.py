@@ -135,3 +135,49 @@ class W8A8BFP32OFP32Linear(_Int8Linear):
         q.a = _scale_tensor(input_scale * weight_scale)
         q.input_scale, q.weight_scale = input_scale, weight_scale
         return q
+
+
+class DynamicW8A8BFP32OFP32Linear(torch.nn.Module):
+    """fc2 / out_proj with the activation quantised on the fly, per tensor (reference:
+    nn/linear.py:281-342, `DanymicW8A8BFP32OFP32Linear`).  The reference's forward cannot run (it
+    names an attribute that does not exist and registers `weight_scale` twice); this is the
+    arithmetic it spells out: `x8, s = quantize_per_tensor_absmax(x)`, then
+    `linear_a8_w8_bfp32_ofp32(x8, weight, bias, s * weight_scale, 1)`.  The scale stays a device
+    tensor (no host synchronisation) and, unlike the helper, the caller's `x` is left untouched."""
+
+    def __init__(self, in_features, out_features, alpha=1.0, beta=1.0):
+        super().__init__()
+        self.in_features, self.out_features = in_features, out_features
+        self.register_buffer("weight", torch.randint(-127, 127, (out_features, in_features), dtype=torch.int8))
+        self.register_buffer("bias", torch.zeros(out_features, dtype=torch.float32))
+        self.register_buffer("weight_scale", torch.tensor(alpha, dtype=torch.float32))
+        self.register_buffer("b", torch.tensor(1.0, dtype=torch.float32))
+
+    def _apply(self, fn, *args, **kwargs):
+        super()._apply(fn, *args, **kwargs)
+        for name in ("bias", "weight_scale", "b"):  # what the kernel reads as fp32 stays fp32 under .half()
+            t = getattr(self, name)
+            if t.dtype != torch.float32:
+                setattr(self, name, t.to(torch.float32))
+        return self
+
+    @torch.no_grad()
+    def forward(self, x):
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, x.shape[-1])
+        scale = x2.abs().max() / 127                        # quantize_per_tensor_absmax (functional/quantization.py:5-14)
+        x8 = (x2 / scale).round_().to(torch.int8)
+        alpha = (scale.to(torch.float32) * self.weight_scale).to(torch.float32)
+        y = linear_a8_w8_bfp32_ofp32(x8, self.weight, self.bias, alpha, self.b)
+        return y.view(*lead, -1)
+
+    @classmethod
+    def from_float(cls, module: torch.nn.Linear):
+        q = cls(module.in_features, module.out_features)
+        q.weight, weight_scale = quantize_per_tensor_absmax(module.weight)
+        q.bias = module.bias.to(torch.float32)
+        q.weight_scale = weight_scale.to(torch.float32).reshape(())
+        return q
+
+
+DanymicW8A8BFP32OFP32Linear = DynamicW8A8BFP32OFP32Linear  # the reference's spelling (nn/linear.py:281)
