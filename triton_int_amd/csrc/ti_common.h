@@ -65,10 +65,8 @@ __device__ __forceinline__ float gelu_tanh_scaled(float x, float scale) {
 }
 
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-  unsigned u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+  __bf16 h = (__bf16)f;  // v_cvt_pk_bf16_f32, round-to-nearest-even
+  return __builtin_bit_cast(uint16_t, h);
 }
 
 __device__ __forceinline__ uint16_t f32_to_f16_bits(float f) {
