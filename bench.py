@@ -258,7 +258,9 @@ def extras(torch, dev):
     sc = torch.empty((B, S, S), dtype=torch.int8, device=dev)
     ms = time_region(torch, lambda: bmm.bmm_s8t_s8n_s8t(q, k, 1e-3, out=sc), 10, 2)
     out["bmm_qk_s8_160x2048x2048x128"] = {"ms": ms, "GBps": 755.0e6 / ms / 1e6, "TOPS": 171.8e9 / ms / 1e9}
-    p = torch.randint(0, 128, (B, S, S), dtype=torch.int8, device=dev)
+    # probabilities as the baseline prescribes them: round(127 * softmax(N(0,1) * s)), here from this
+    # library's own softmax-quantise kernel on int8 scores round(32 * N(0,1)) with scale 0.05 (logit std 1.6)
+    p = fused.softmax_q(torch.randn((B, S, S), device=dev).mul_(32).round_().clamp_(-127, 127).to(torch.int8), 0.05)
     vt = torch.randint(-127, 128, (B, D, S), dtype=torch.int8, device=dev)
     of = torch.empty((B, S, D), dtype=torch.float32, device=dev)
     ms = time_region(torch, lambda: bmm.bmm_s8t_s8n_f32t(p, vt, 1.0 / 16129, out=of), 10, 2)
