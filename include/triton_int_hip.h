@@ -222,6 +222,19 @@ int ti_transpose_i8(const int8_t* src, int64_t src_row_stride, int8_t* dst, int6
                     int rows, int cols, void* stream);
 
 /*
+ * W8A8BFP32OFP32Linear (nn/linear.py:222-278) followed by the residual add its caller performs
+ * (`fc2(x) + residual` in a decoder layer):
+ *     C[m][n] = (alpha * f(acc[m][n]) + beta * bias[n]) + residual[m][n]        fp32, rounded per step
+ * A [M,K], W [N,K] int8 with unit column stride, bias fp32 [N] or NULL, residual and C fp32 with unit
+ * column stride (row strides in elements).  With M <= 16 the weight-streaming decode kernel adds the
+ * residual as it stores (one launch instead of two); otherwise the GEMM is followed by an add kernel.
+ * Same bits as the linear followed by an fp32 add.  C must not overlap the residual.
+ */
+int ti_linear_i8_residual_f32(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw, const float* bias,
+                              const float* alpha, const float* beta, const float* residual, int64_t ldr,
+                              float* C, int64_t ldc, int M, int N, int K, void* stream);
+
+/*
  * Appends S new positions to an int8 KV cache in one launch: K [S, heads*D] (row stride
  * k_src_row_stride) is copied to k_dst[h][s][d] = k_dst + h * k_head_stride + s * D + d (k_dst points at
  * the first new slot of head 0 in a [heads, T, D] cache, k_head_stride = T * D), and V [S, heads*D]

@@ -67,6 +67,8 @@ def test_decoder_layer_prefill_and_decode_small():
     out = layer(gpu(hidden), _trace=tr)
     assert out.shape == (B, S, H) and out.dtype == torch.float32
     _check_stages(layer, tr, hidden, B, S, causal_q_len=S)
+    # untraced, fc2 and the residual add are one library call: same bits
+    assert torch.equal(layer(gpu(hidden)), out)
     # the one-kernel attention forced on for this small two-batch case: same context rows
     layer.fused_attention_min_queries = 1
     trf = {}
@@ -87,6 +89,8 @@ def test_decoder_layer_prefill_and_decode_small():
     assert out.shape == (B, Sd, H)
     assert torch.equal(k_cache[:, :T - Sd], k_old[:, :T - Sd]) and torch.equal(vt_cache[:, :, :T - Sd], vt_old[:, :, :T - Sd])
     _check_stages(layer, tr, hidden_d, B, Sd, causal_q_len=Sd)
+    k3, v3 = k_old.clone(), vt_old.clone()
+    assert torch.equal(layer(gpu(hidden_d), kv_cache=(k3, v3)), out)  # decode: the GEMM kernel adds the residual
     # the same decode step through the one-kernel attention, the default for 16 or fewer query rows
     # (cache offset T - S in the causal mask)
     layer.fused_attention = True

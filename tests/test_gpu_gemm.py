@@ -474,3 +474,27 @@ def test_decode_kernel_several_passes_strided_and_16bit_outputs():
     for dt, odt in ((torch.float16, O.DT_F16), (torch.bfloat16, O.DT_BF16)):
         got16 = cpu(linear.linear_a8_w8_bfp32_ofp32(ga, gw, gpu(bf), alpha, 1.0, dtype=dt))
         assert np.array_equal(got16, O.linear_a8_w8_bfp32_ofp32(a, w, bf, alpha, 1.0, out_dtype=odt))
+
+
+@pytest.mark.parametrize("M,N,K", [(16, 5120, 20480), (1, 272, 1040), (7, 5124, 1024), (300, 320, 256), (2048, 768, 512), (16, 50272, 1024)])
+def test_linear_with_residual_equals_linear_then_add(M, N, K):
+    """ti_linear_i8_residual_f32: the decode kernel's fused add (M <= 16) and the GEMM + add-kernel pair
+    give the bits of the fp32 linear followed by an fp32 add."""
+    linear, _, _ = _kl()
+    g = rng(M + N + K)
+    a, w = rand_i8(g, M, K), rand_i8(g, N, K)
+    bf = g.standard_normal(N).astype(np.float32)
+    res = (g.standard_normal((M, N)) * 3).astype(np.float32)
+    alpha = np.float32(40.0 / (np.sqrt(K) * 127 * 127 / 3))
+    want = O.linear_a8_w8_bfp32_ofp32(a, w, bf, alpha, 1.0) + res
+    ga, gw, gb, gr = gpu(a), gpu(w), gpu(bf), gpu(res)
+    got = linear.linear_a8_w8_bfp32_ofp32_residual(ga, gw, gb, alpha, 1.0, gr)
+    assert got.dtype == torch.float32 and np.array_equal(cpu(got), want)
+    assert np.array_equal(cpu(gr), res)  # the residual is left alone
+    # into a given buffer, without a bias; an output that is the residual itself is refused
+    buf = torch.empty((M, N), dtype=torch.float32, device=DEV)
+    got2 = linear.linear_a8_w8_bfp32_ofp32_residual(ga, gw, None, alpha, 1.0, gr, out=buf)
+    assert got2.data_ptr() == buf.data_ptr()
+    assert np.array_equal(cpu(buf), O.linear_a8_w8_ofp32(a, w, alpha) + res)
+    with pytest.raises(AssertionError):
+        linear.linear_a8_w8_bfp32_ofp32_residual(ga, gw, None, alpha, 1.0, gr, out=gr)

@@ -39,6 +39,9 @@ struct GemmParams {
   // bias elements [b * bias_bs, b * bias_bs + N) and the scalars alpha[b * scale_bs], beta[b * scale_bs]
   int64_t bias_bs;
   int64_t scale_bs;
+  // fp32 outputs of gemm_rows4_kernel only: C = epilogue value + resid[m * resid_rs + n]
+  const float* resid;
+  int64_t resid_rs;
 };
 
 enum OutClass { OUT8 = 0, OUT32 = 1, OUT16 = 2 };
@@ -1453,7 +1456,7 @@ constexpr int R4_NW = 8, R4_RG = 4, R4_KC = 1024, R4_PITCH = R4_KC + 16, R4_WPIT
 template <int OUTCLS>
 __device__ __attribute__((noinline)) void rows4_store_tile(const EpiCtx e, char* Cz, int64_t sCm, int64_t sCn, int M, int N,
                                                           int out_dtype, unsigned tile0, int tid, int unit0, int u_end,
-                                                          int max_units) {
+                                                          int max_units, const float* resid, int64_t resid_rs) {
   constexpr int ESZ = OUTCLS == OUT8 ? 1 : (OUTCLS == OUT32 ? 4 : 2);
   constexpr int RING = R4_NST * R4_RG * R4_WPITCH;
   const int row = tid >> 5, grp = tid & 31;
@@ -1468,6 +1471,9 @@ __device__ __attribute__((noinline)) void rows4_store_tile(const EpiCtx e, char*
     const int n = min(n0 + i, N - 1);
     const int bias_i32 = (e.epilogue == TI_EPI_I32 && e.bias_kind == TI_BIAS_I32) ? ((const int*)e.bias)[n] : 0;
     b[i] = convert_one<OUTCLS>(e, a[i], column_term(e, n), bias_i32, out_dtype);
+    if constexpr (OUTCLS == OUT32) {
+      if (resid) b[i] = __float_as_uint(__uint_as_float(b[i]) + resid[(int64_t)row * resid_rs + n]);  // fp32 epilogues only (host)
+    }
   }
   char* dst = Cz + ((int64_t)row * sCm + (int64_t)n0 * sCn) * ESZ;
   if (sCn == 1 && n0 + R4_RG <= N && (((uintptr_t)dst) & (R4_RG * ESZ - 1)) == 0) {
@@ -1635,7 +1641,7 @@ __global__ __launch_bounds__((R4_NW + 1) * 64) void gemm_rows4_kernel(GemmParams
     }
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     rows4_store_tile<OUTCLS>(e, Cz, p.sCm, p.sCn, p.M, p.N, p.out_dtype, lds_base + R4_XB * XBUF + 2 * STAGE, tid,
-                             ub0 + pass * (NSLOT * R4_UMAX), u_end, NSLOT * R4_UMAX);
+                             ub0 + pass * (NSLOT * R4_UMAX), u_end, NSLOT * R4_UMAX, p.resid, p.resid_rs);
   }
 }
 
@@ -1911,6 +1917,51 @@ static int run(GemmParams p, int config, hipStream_t stream) {
 
 }  // namespace ti
 
+namespace ti {
+
+// C[m][n] += R[m][n] for fp32 row-major matrices (unit column stride): the second launch of a linear
+// with a residual when the GEMM kernel that ran does not add it itself.
+__global__ __launch_bounds__(256) void add_rows_f32_kernel(float* C, int64_t ldc, const float* R, int64_t ldr, int M, int N, int vec) {
+  const int64_t per_row = vec ? N / 4 : N;
+  const int64_t total = (int64_t)M * per_row;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    const int64_t m = i / per_row, c = i - m * per_row;
+    if (vec) {
+      v4f* d = (v4f*)(C + m * ldc) + c;
+      *d = *d + *((const v4f*)(R + m * ldr) + c);
+    } else {
+      C[m * ldc + c] += R[m * ldr + c];
+    }
+  }
+}
+
+static int run_with_residual(GemmParams p, const float* R, int64_t ldr, hipStream_t stream) {
+  int rc = validate(p);
+  if (rc != TI_OK) return rc;
+  if (p.M == 0 || p.N == 0) return TI_OK;
+  if (!R) return fail(TI_E_NULL, "residual is NULL");
+  if ((const void*)R == (const void*)p.C) return fail(TI_E_STRIDE, "the output must not alias the residual");
+  if (ldr < p.N || p.sCn != 1 || p.sCm < p.N) return fail(TI_E_STRIDE, "residual and output rows must be contiguous and cover a row");
+  rc = check_device();
+  if (rc != TI_OK) return rc;
+  if (!p.bias) p.bias_kind = TI_BIAS_NONE;
+  const int cfg = pick_config(p);
+  if (g_configs[cfg].rows4) {  // the decode kernel adds the residual in its store phase
+    p.resid = R;
+    p.resid_rs = ldr;
+    return run(p, cfg, stream);
+  }
+  rc = run(p, cfg, stream);
+  if (rc != TI_OK) return rc;
+  const int vec = (p.N % 4 == 0) && (p.sCm % 4 == 0) && (ldr % 4 == 0) && (((uintptr_t)p.C | (uintptr_t)R) & 15) == 0;
+  const int64_t items = (int64_t)p.M * (vec ? p.N / 4 : p.N);
+  const unsigned blocks = (unsigned)(items / 256 + 1 < 256 * 16 ? items / 256 + 1 : 256 * 16);
+  add_rows_f32_kernel<<<dim3(blocks), dim3(256), 0, stream>>>((float*)p.C, p.sCm, R, ldr, p.M, p.N, vec);
+  return launch_status("add_rows_f32_kernel");
+}
+
+}  // namespace ti
+
 extern "C" {
 
 int ti_bmm_i8_config(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk, const int8_t* B, int64_t sBb,
@@ -1928,6 +1979,7 @@ int ti_bmm_i8_config(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk, con
   p.epilogue = epilogue; p.out_dtype = out_dtype; p.round_mode = round_mode;
   p.tiles_m = p.tiles_n = 0; p.group_m = 1; p.ksplit = 1;
   p.bias_bs = 0; p.scale_bs = 0;
+  p.resid = nullptr; p.resid_rs = 0;
   return ti::run(p, config, (hipStream_t)stream);
 }
 
@@ -1948,6 +2000,7 @@ int ti_bmm_i8_grouped(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk, co
   p.epilogue = epilogue; p.out_dtype = out_dtype; p.round_mode = round_mode;
   p.tiles_m = p.tiles_n = 0; p.group_m = 1; p.ksplit = 1;
   p.bias_bs = bias_batch_stride; p.scale_bs = scale_batch_stride;
+  p.resid = nullptr; p.resid_rs = 0;
   return ti::run(p, config, (hipStream_t)stream);
 }
 
@@ -1957,6 +2010,24 @@ int ti_bmm_i8(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk, const int8
               int round_mode, void* stream) {
   return ti_bmm_i8_config(A, sAb, sAm, sAk, B, sBb, sBn, sBk, C, sCb, sCm, sCn, batch, M, N, K, bias, bias_kind,
                           alpha, beta, epilogue, out_dtype, round_mode, -1, stream);
+}
+
+int ti_linear_i8_residual_f32(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw, const float* bias,
+                              const float* alpha, const float* beta, const float* residual, int64_t ldr, float* C,
+                              int64_t ldc, int M, int N, int K, void* stream) {
+  ti::GemmParams p;
+  p.A = A; p.B = W; p.C = C;
+  p.sAb = 0; p.sAm = lda; p.sAk = 1;
+  p.sBb = 0; p.sBn = ldw; p.sBk = 1;
+  p.sCb = 0; p.sCm = ldc; p.sCn = 1;
+  p.batch = 1; p.M = M; p.N = N; p.K = K;
+  p.bias = bias; p.bias_kind = bias ? TI_BIAS_F32 : TI_BIAS_NONE;
+  p.alpha = alpha; p.beta = beta;
+  p.epilogue = TI_EPI_SCALE_F; p.out_dtype = TI_F32; p.round_mode = TI_ROUND_RNE_CLAMP;
+  p.tiles_m = p.tiles_n = 0; p.group_m = 1; p.ksplit = 1;
+  p.bias_bs = 0; p.scale_bs = 0;
+  p.resid = nullptr; p.resid_rs = 0;
+  return ti::run_with_residual(p, residual, ldr, (hipStream_t)stream);
 }
 
 #ifdef TI_TRACE

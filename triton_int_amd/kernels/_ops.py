@@ -49,6 +49,10 @@ _OPS = {
         "(Tensor a, Tensor b, Tensor? bias, Tensor scale_a, Tensor scale_b) -> Tensor",
         lambda a, b, bias, sa, sb: _linear.linear_a8_w8_bfp32_ofp32(a, b, bias, sa, sb, dtype=torch.float32),
         lambda a, b, bias, sa, sb: _lin_out(a, b, torch.float32)),
+    "linear_a8_w8_bfp32_ofp32_residual": (
+        "(Tensor a, Tensor b, Tensor? bias, Tensor scale_a, Tensor scale_b, Tensor residual) -> Tensor",
+        lambda a, b, bias, sa, sb, r: _linear.linear_a8_w8_bfp32_ofp32_residual(a, b, bias, sa, sb, r),
+        lambda a, b, bias, sa, sb, r: _lin_out(a, b, torch.float32)),
     "linear_a8_w8_ofp32": (
         "(Tensor a, Tensor b, Tensor scale) -> Tensor",
         lambda a, b, s: _linear.linear_a8_w8_ofp32(a, b, s),

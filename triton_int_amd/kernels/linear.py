@@ -64,3 +64,42 @@ def linear_a8_w8_bfp32_ofp32(a, b, bias, scale_a, scale_b, out=None, dtype=None,
         bias = bias.to(torch.float32)
     return _linear(a, b, epilogue=L.EPI_SCALE_F, out_dtype=dtype, bias=bias, alpha=scale_a, beta=scale_b, out=out,
                    config=_config)
+
+
+def linear_a8_w8_bfp32_ofp32_residual(a, b, bias, scale_a, scale_b, residual, out=None):
+    """`linear_a8_w8_bfp32_ofp32(a, b, bias, scale_a, scale_b) + residual` in fp32 as one library call
+    (reference: kernels/linear.py:819-853 followed by the caller's add): with 16 or fewer rows the
+    decode kernel adds the residual while it stores, otherwise an add kernel follows the GEMM.
+    `out` must not overlap `residual`."""
+    L.require_cuda(a, b, bias, residual, out)
+    assert a.dtype == torch.int8 and b.dtype == torch.int8, "operands must be int8"
+    assert len(b.shape) == 2 and a.shape[-1] == b.shape[1], "Incompatible dimensions"
+    N, K = b.shape
+    lead = a.shape[:-1]
+    a2 = a.reshape(-1, K)
+    M = a2.shape[0]
+    assert residual.dtype == torch.float32 and residual.numel() == M * N, "residual must be fp32 [*, N]"
+    r2 = residual.reshape(M, N)
+    if a2.stride(1) != 1:
+        a2 = a2.contiguous()
+    if r2.stride(1) != 1:
+        r2 = r2.contiguous()
+    if b.stride(1) != 1:
+        b = b.contiguous()
+    if bias is not None:
+        assert bias.numel() == N
+        bias = bias.to(torch.float32).contiguous()
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.float32, device=a.device)
+    else:
+        assert out.dtype == torch.float32 and out.numel() == M * N and out.is_contiguous()
+    o2 = out.view(M, N)
+    dev = a.device
+    alpha, beta = L.scale_tensor(scale_a, dev), L.scale_tensor(scale_b, dev)
+    with L.on_device(dev):
+        rc = L.lib().ti_linear_i8_residual_f32(a2.data_ptr(), a2.stride(0) if M > 1 else K, b.data_ptr(), b.stride(0),
+                                               L.ptr(bias), alpha.data_ptr(), beta.data_ptr(), r2.data_ptr(),
+                                               r2.stride(0) if M > 1 else N, o2.data_ptr(), N, M, N, K,
+                                               L.current_stream(dev))
+    L.check(rc, "ti_linear_i8_residual_f32")
+    return o2.view(*lead, N)

@@ -14,6 +14,7 @@ from ..kernels.linear import (
     linear_a8_w8_b32_o32,
     linear_a8_w8_b32_o32_with_scaling,
     linear_a8_w8_bfp32_ofp32,
+    linear_a8_w8_bfp32_ofp32_residual,
     linear_relu_a8_w8_b8_o8,
 )
 
@@ -126,6 +127,14 @@ class W8A8BFP32OFP32Linear(_Int8Linear):
 
     def _launch(self, x):
         return linear_a8_w8_bfp32_ofp32(x, self.weight, self.bias, self.a, self.b)
+
+    @torch.no_grad()
+    def forward_add(self, x, residual):
+        """forward(x) + residual (fp32, same shape as the output) as one library call."""
+        lead = x.shape[:-1]
+        y = linear_a8_w8_bfp32_ofp32_residual(x.view(-1, x.shape[-1]), self.weight, self.bias, self.a, self.b,
+                                              residual.reshape(-1, self.out_features))
+        return y.view(*lead, -1)
 
     @classmethod
     def from_float(cls, module: torch.nn.Linear, input_scale):

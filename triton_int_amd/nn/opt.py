@@ -17,6 +17,7 @@ end-to-end tests: every heavy step is one of the package's HIP kernels, torch on
       resid, h8 = DQ_Add_LayerNorm_Q(hidden, acc)           (ti_dq_add_layernorm_q)
       f8     = W8A8BFP32OFP32_GeLu_Q(h8) -> int8            (GEMM + GELU-quant epilogue)   fc1
       out    = W8A8BFP32OFP32Linear(f8) + resid -> fp32                                  fc2
+               (one library call, ti_linear_i8_residual_f32: in decode the GEMM kernel adds the residual)
 """
 from __future__ import annotations
 
@@ -51,6 +52,9 @@ class W8A8OPTDecoderLayer(torch.nn.Module):
         # rows per head); the three-launch chain in between (too few workgroups for the block kernel)
         self.fused_attention = True
         self.fused_attention_min_queries = 128
+        # fc2 and the residual add that follows it as one library call (a traced forward keeps them apart
+        # so that the fc2 output can be inspected)
+        self.fused_residual = True
 
     @torch.no_grad()
     def randomize(self, seed=0):
@@ -172,10 +176,15 @@ class W8A8OPTDecoderLayer(torch.nn.Module):
         mark("ln2_dq_add_layernorm_q")
         f8 = self.fc1(h8b)
         mark("fc1_linear_gelu_q")
-        y = self.fc2(f8)
-        mark("fc2_linear_f32")
-        out = y + resid
-        mark("residual_add")
+        if self.fused_residual and _trace is None:
+            y = None
+            out = self.fc2.forward_add(f8, resid)   # decode: one launch; prefill: GEMM + add kernel
+            mark("fc2_linear_f32_plus_residual")
+        else:
+            y = self.fc2(f8)
+            mark("fc2_linear_f32")
+            out = y + resid
+            mark("residual_add")
         if _trace is not None:
             _trace.update(h8=h8, q=q, k_all=k_all, vt_all=vt_all, scores=scores, probs=probs, ctx=ctx, acc=acc,
                           resid=resid, h8b=h8b, f8=f8, fc2=y, out=out)
