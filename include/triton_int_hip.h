@@ -235,6 +235,21 @@ int ti_linear_i8_residual_f32(const int8_t* A, int64_t lda, const int8_t* W, int
                               float* C, int64_t ldc, int M, int N, int K, void* stream);
 
 /*
+ * A decode step's q / k / v projections (three W8A8B8O8Linear of one input, nn/linear.py:18-67) with the
+ * KV-cache append folded in: one launch of the weight-streaming kernel instead of ti_bmm_i8_grouped
+ * followed by ti_kv_append_i8.  A [M,K] (M <= 16, K >= 1024), W [3N,K] the stacked weights, bias int8
+ * [3N] or NULL, alpha3 / beta3 fp32 [3], C [M,3N] int8 (row stride ldc) receives q | k | v as
+ * ti_bmm_i8_grouped writes them; in addition k goes to k_dst[h * k_head_stride + m * D + d] and v to
+ * vt_dst[(h * D + d) * vt_row_stride + m] (k_dst / vt_dst point at the first new slot / column, as for
+ * ti_kv_append_i8; N = heads * D, D % 16 == 0).  TI_E_COMBO when the operands do not fit the kernel
+ * (the caller then makes the two calls).
+ */
+int ti_qkv_decode_i8(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw, const int8_t* bias,
+                     const float* alpha3, const float* beta3, int8_t* C, int64_t ldc, int M, int N, int K,
+                     int8_t* k_dst, int64_t k_head_stride, int8_t* vt_dst, int64_t vt_row_stride, int D,
+                     void* stream);
+
+/*
  * Appends S new positions to an int8 KV cache in one launch: K [S, heads*D] (row stride
  * k_src_row_stride) is copied to k_dst[h][s][d] = k_dst + h * k_head_stride + s * D + d (k_dst points at
  * the first new slot of head 0 in a [heads, T, D] cache, k_head_stride = T * D), and V [S, heads*D]

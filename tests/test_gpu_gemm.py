@@ -498,3 +498,36 @@ def test_linear_with_residual_equals_linear_then_add(M, N, K):
     assert np.array_equal(cpu(buf), O.linear_a8_w8_ofp32(a, w, alpha) + res)
     with pytest.raises(AssertionError):
         linear.linear_a8_w8_bfp32_ofp32_residual(ga, gw, None, alpha, 1.0, gr, out=gr)
+
+
+@pytest.mark.parametrize("S,heads,D,K,T", [(16, 40, 128, 5120, 2048), (1, 8, 64, 1024, 40), (7, 3, 128, 2064, 96), (16, 5, 16, 1040, 16)])
+def test_qkv_decode_with_kv_append_equals_grouped_linear_plus_append(S, heads, D, K, T):
+    """ti_qkv_decode_i8: projections identical to the grouped launch (hence to three separate linears),
+    caches identical to numpy indexing; cache positions before the last S are untouched."""
+    linear, _, _ = _kl()
+    g = rng(S * 3 + heads + K)
+    N = heads * D
+    a, w3 = rand_i8(g, S, K), rand_i8(g, 3 * N, K)
+    b3 = rand_i8(g, 3 * N)
+    al = (g.uniform(0.5, 1.5, 3) * 40.0 / (np.sqrt(K) * 127 * 127 / 3)).astype(np.float32)
+    be = g.uniform(0.01, 0.1, 3).astype(np.float32)
+    k_cache = g.integers(-128, 128, size=(heads, T, D), dtype=np.int8)
+    vt_cache = g.integers(-128, 128, size=(heads, D, T), dtype=np.int8)
+    want = np.concatenate([O.linear_a8_w8_b8_o8(a, w3[i * N:(i + 1) * N], b3[i * N:(i + 1) * N], al[i], be[i]) for i in range(3)], axis=1)
+    want_k, want_vt = k_cache.copy(), vt_cache.copy()
+    want_k[:, T - S:, :] = want[:, N:2 * N].reshape(S, heads, D).transpose(1, 0, 2)
+    want_vt[:, :, T - S:] = want[:, 2 * N:].reshape(S, heads, D).transpose(1, 2, 0)
+    gk, gvt = gpu(k_cache), gpu(vt_cache)
+    got = linear.linear_qkv_decode_a8_w8_b8_o8(gpu(a), gpu(w3), gpu(b3), gpu(al), gpu(be), gk, gvt)
+    assert got is not None and np.array_equal(cpu(got), want)
+    assert np.array_equal(cpu(gk), want_k) and np.array_equal(cpu(gvt), want_vt)
+
+
+def test_qkv_decode_declines_what_the_decode_kernel_cannot_take():
+    linear, _, _ = _kl()
+    g = rng(1)
+    a, w3, b3 = rand_i8(g, 32, 1024), rand_i8(g, 3 * 128, 1024), rand_i8(g, 3 * 128)
+    s3 = gpu(np.ones(3, np.float32))
+    kc, vc = gpu(np.zeros((1, 64, 128), np.int8)), gpu(np.zeros((1, 128, 64), np.int8))
+    assert linear.linear_qkv_decode_a8_w8_b8_o8(gpu(a), gpu(w3), gpu(b3), s3, s3, kc, vc) is None       # 32 rows
+    assert linear.linear_qkv_decode_a8_w8_b8_o8(gpu(a[:4, :512].copy()), gpu(w3[:, :512].copy()), gpu(b3), s3, s3, kc, vc) is None  # K < 1024

@@ -26,7 +26,7 @@ TORCH_TO_BIAS = {torch.int8: BIAS_I8, torch.int32: BIAS_I32, torch.float32: BIAS
 
 EXPORTS = ("ti_version", "ti_last_error", "ti_mfma_i8_probe", "ti_bmm_i8", "ti_bmm_i8_config", "ti_bmm_i8_grouped", "ti_gemm_num_configs",
            "ti_gemm_config_name", "ti_gemm_last_config", "ti_layernorm_q", "ti_dq_add_layernorm_q", "ti_gelu_q", "ti_softmax_q", "ti_transpose_i8", "ti_attention_i8", "ti_quantize_per_token_absmax", "ti_kv_append_i8",
-           "ti_layernorm_fp", "ti_linear_i8_residual_f32")
+           "ti_layernorm_fp", "ti_linear_i8_residual_f32", "ti_qkv_decode_i8")
 
 _lib = None
 
@@ -76,6 +76,9 @@ def _declare(lib):
                                     _int, _int, _int, _int, _f32, _f32, _f32, _int, _vp]
     lib.ti_linear_i8_residual_f32.restype = _int
     lib.ti_linear_i8_residual_f32.argtypes = [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _int, _int, _int, _vp]
+    lib.ti_qkv_decode_i8.restype = _int
+    lib.ti_qkv_decode_i8.argtypes = [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _int, _int, _int,
+                                     _vp, _i64, _vp, _i64, _int, _vp]
     lib.ti_gelu_q.restype = _int
     lib.ti_gelu_q.argtypes = [_vp, _vp, _vp, _i64, _int, _vp]
 

@@ -42,6 +42,12 @@ struct GemmParams {
   // fp32 outputs of gemm_rows4_kernel only: C = epilogue value + resid[m * resid_rs + n]
   const float* resid;
   int64_t resid_rs;
+  // int8 outputs of a grouped q/k/v launch of gemm_rows4_kernel only: batch 1 (k) also goes to
+  // kv_k[head * kv_k_hs + m * kv_D + d], batch 2 (v) to kv_vt[(head * kv_D + d) * kv_vt_rs + m]
+  int8_t* kv_k;
+  int8_t* kv_vt;
+  int64_t kv_k_hs, kv_vt_rs;
+  int kv_D;
 };
 
 enum OutClass { OUT8 = 0, OUT32 = 1, OUT16 = 2 };
@@ -1456,7 +1462,8 @@ constexpr int R4_NW = 8, R4_RG = 4, R4_KC = 1024, R4_PITCH = R4_KC + 16, R4_WPIT
 template <int OUTCLS>
 __device__ __attribute__((noinline)) void rows4_store_tile(const EpiCtx e, char* Cz, int64_t sCm, int64_t sCn, int M, int N,
                                                           int out_dtype, unsigned tile0, int tid, int unit0, int u_end,
-                                                          int max_units, const float* resid, int64_t resid_rs) {
+                                                          int max_units, const float* resid, int64_t resid_rs, int bz,
+                                                          const GemmParams* kp) {
   constexpr int ESZ = OUTCLS == OUT8 ? 1 : (OUTCLS == OUT32 ? 4 : 2);
   constexpr int RING = R4_NST * R4_RG * R4_WPITCH;
   const int row = tid >> 5, grp = tid & 31;
@@ -1476,6 +1483,22 @@ __device__ __attribute__((noinline)) void rows4_store_tile(const EpiCtx e, char*
     }
   }
   char* dst = Cz + ((int64_t)row * sCm + (int64_t)n0 * sCn) * ESZ;
+  if constexpr (OUTCLS == OUT8) {
+    if (bz > 0 && n0 + R4_RG <= N) {
+      // KV-cache append of a decode step's k / v projections; the fields are read through kp, the
+      // kernel's own argument block (the builtin that returns it yields null outside a kernel, so
+      // the kernel passes it along)
+      if (kp->kv_k) {
+        const int D = kp->kv_D, head = n0 / D, d = n0 - head * D;
+        if (bz == 1) {
+          *(unsigned*)(kp->kv_k + (int64_t)head * kp->kv_k_hs + (int64_t)row * D + d) = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
+        } else if (bz == 2) {
+#pragma unroll
+          for (int i = 0; i < R4_RG; ++i) kp->kv_vt[(int64_t)(n0 + i) * kp->kv_vt_rs + row] = (int8_t)b[i];
+        }
+      }
+    }
+  }
   if (sCn == 1 && n0 + R4_RG <= N && (((uintptr_t)dst) & (R4_RG * ESZ - 1)) == 0) {
     if constexpr (OUTCLS == OUT8) *(unsigned*)dst = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
     else if constexpr (OUTCLS == OUT32) *(v4u*)dst = (v4u){b[0], b[1], b[2], b[3]};
@@ -1641,7 +1664,8 @@ __global__ __launch_bounds__((R4_NW + 1) * 64) void gemm_rows4_kernel(GemmParams
     }
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     rows4_store_tile<OUTCLS>(e, Cz, p.sCm, p.sCn, p.M, p.N, p.out_dtype, lds_base + R4_XB * XBUF + 2 * STAGE, tid,
-                             ub0 + pass * (NSLOT * R4_UMAX), u_end, NSLOT * R4_UMAX, p.resid, p.resid_rs);
+                             ub0 + pass * (NSLOT * R4_UMAX), u_end, NSLOT * R4_UMAX, p.resid, p.resid_rs, bz,
+                             (const GemmParams*)__builtin_amdgcn_kernarg_segment_ptr());
   }
 }
 
@@ -1980,6 +2004,7 @@ int ti_bmm_i8_config(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk, con
   p.tiles_m = p.tiles_n = 0; p.group_m = 1; p.ksplit = 1;
   p.bias_bs = 0; p.scale_bs = 0;
   p.resid = nullptr; p.resid_rs = 0;
+  p.kv_k = p.kv_vt = nullptr; p.kv_k_hs = p.kv_vt_rs = 0; p.kv_D = 1;
   return ti::run(p, config, (hipStream_t)stream);
 }
 
@@ -2001,7 +2026,39 @@ int ti_bmm_i8_grouped(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk, co
   p.tiles_m = p.tiles_n = 0; p.group_m = 1; p.ksplit = 1;
   p.bias_bs = bias_batch_stride; p.scale_bs = scale_batch_stride;
   p.resid = nullptr; p.resid_rs = 0;
+  p.kv_k = p.kv_vt = nullptr; p.kv_k_hs = p.kv_vt_rs = 0; p.kv_D = 1;
   return ti::run(p, config, (hipStream_t)stream);
+}
+
+int ti_qkv_decode_i8(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw, const int8_t* bias,
+                     const float* alpha3, const float* beta3, int8_t* C, int64_t ldc, int M, int N, int K,
+                     int8_t* k_dst, int64_t k_head_stride, int8_t* vt_dst, int64_t vt_row_stride, int D,
+                     void* stream) {
+  using namespace ti;
+  if (M > 16 || K < 1024 || D <= 0 || (D & 15) || N % D) return fail(TI_E_COMBO, "needs M <= 16, K >= 1024, D %% 16 == 0, N %% D == 0");
+  if (!k_dst || !vt_dst) return fail(TI_E_NULL, "k_dst and vt_dst are required");
+  if (((uintptr_t)k_dst & 3) || (k_head_stride & 3)) return fail(TI_E_STRIDE, "k_dst and its head stride must be multiples of 4 bytes");
+  GemmParams p;
+  p.A = A; p.B = W; p.C = C;
+  p.sAb = 0; p.sAm = lda; p.sAk = 1;
+  p.sBb = (int64_t)N * ldw; p.sBn = ldw; p.sBk = 1;
+  p.sCb = N; p.sCm = ldc; p.sCn = 1;
+  p.batch = 3; p.M = M; p.N = N; p.K = K;
+  p.bias = bias; p.bias_kind = bias ? TI_BIAS_I8 : TI_BIAS_NONE;
+  p.alpha = alpha3; p.beta = beta3;
+  p.epilogue = TI_EPI_SCALE_I8; p.out_dtype = TI_I8; p.round_mode = TI_ROUND_RNE_CLAMP;
+  p.tiles_m = p.tiles_n = 0; p.group_m = 1; p.ksplit = 1;
+  p.bias_bs = N; p.scale_bs = 1;
+  p.resid = nullptr; p.resid_rs = 0;
+  p.kv_k = k_dst; p.kv_vt = vt_dst; p.kv_k_hs = k_head_stride; p.kv_vt_rs = vt_row_stride; p.kv_D = D;
+  int rc = validate(p);
+  if (rc != TI_OK) return rc;
+  if (M == 0 || N == 0) return TI_OK;
+  rc = check_device();
+  if (rc != TI_OK) return rc;
+  const int cfg = pick_config(p);
+  if (!g_configs[cfg].rows4) return fail(TI_E_COMBO, "operands not eligible for the decode kernel (16-byte aligned, K-contiguous)");
+  return run(p, cfg, (hipStream_t)stream);
 }
 
 int ti_bmm_i8(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk, const int8_t* B, int64_t sBb, int64_t sBn,
@@ -2027,6 +2084,7 @@ int ti_linear_i8_residual_f32(const int8_t* A, int64_t lda, const int8_t* W, int
   p.tiles_m = p.tiles_n = 0; p.group_m = 1; p.ksplit = 1;
   p.bias_bs = 0; p.scale_bs = 0;
   p.resid = nullptr; p.resid_rs = 0;
+  p.kv_k = p.kv_vt = nullptr; p.kv_k_hs = p.kv_vt_rs = 0; p.kv_D = 1;
   return ti::run_with_residual(p, residual, ldr, (hipStream_t)stream);
 }
 

@@ -103,3 +103,35 @@ def linear_a8_w8_bfp32_ofp32_residual(a, b, bias, scale_a, scale_b, residual, ou
                                                L.current_stream(dev))
     L.check(rc, "ti_linear_i8_residual_f32")
     return o2.view(*lead, N)
+
+
+def linear_qkv_decode_a8_w8_b8_o8(a, w3, bias3, scale_a3, scale_b3, k_cache, vt_cache, out=None):
+    """The q / k / v projections of a decode step (`linear_group_a8_w8_b8_o8` with 3 groups) with the
+    KV-cache append folded into the same launch: a [S, K] int8 (S <= 16), w3 [3N, K], bias3 int8 [3N],
+    scale_a3 / scale_b3 fp32 device tensors [3]; k_cache int8 [heads, T, D] and vt_cache int8
+    [heads, D, T] (contiguous, N = heads * D) receive the S new positions in their last S slots.
+    Returns the [S, 3N] int8 projections, or None when the shapes do not fit the decode kernel (the
+    caller then uses `linear_group_a8_w8_b8_o8` and `kv_append_i8`)."""
+    L.require_cuda(a, w3, bias3, scale_a3, scale_b3, k_cache, vt_cache, out)
+    S, K = a.shape
+    N = w3.shape[0] // 3
+    heads, T, D = k_cache.shape
+    if not (S <= 16 and K >= 1024 and heads * D == N and D % 16 == 0 and S <= T and tuple(vt_cache.shape) == (heads, D, T)
+            and k_cache.is_contiguous() and vt_cache.is_contiguous() and a.stride(1) == 1 and w3.is_contiguous()):
+        return None
+    assert a.dtype == w3.dtype == bias3.dtype == k_cache.dtype == vt_cache.dtype == torch.int8
+    assert w3.shape == (3 * N, K) and bias3.numel() == 3 * N
+    for t in (scale_a3, scale_b3):
+        assert t.dtype == torch.float32 and t.numel() == 3 and t.is_contiguous()
+    if out is None:
+        out = torch.empty((S, 3 * N), dtype=torch.int8, device=a.device)
+    assert out.dtype == torch.int8 and tuple(out.shape) == (S, 3 * N) and out.is_contiguous()
+    with L.on_device(a.device):
+        rc = L.lib().ti_qkv_decode_i8(a.data_ptr(), a.stride(0) if S > 1 else K, w3.data_ptr(), K, bias3.data_ptr(),
+                                      scale_a3.data_ptr(), scale_b3.data_ptr(), out.data_ptr(), 3 * N, S, N, K,
+                                      k_cache.data_ptr() + (T - S) * D, T * D, vt_cache.data_ptr() + (T - S), T, D,
+                                      L.current_stream(a.device))
+    if rc == -3:  # TI_E_COMBO: operands not eligible for the decode kernel
+        return None
+    L.check(rc, "ti_qkv_decode_i8")
+    return out

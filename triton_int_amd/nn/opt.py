@@ -25,7 +25,7 @@ import torch
 
 from ..kernels.bmm import bmm_s8t_s8n_s8t
 from ..kernels.fused import attention_i8, kv_append_i8, softmax_q, transpose_i8
-from ..kernels.linear import linear_group_a8_w8_b8_o8
+from ..kernels.linear import linear_group_a8_w8_b8_o8, linear_qkv_decode_a8_w8_b8_o8
 from .fused import DQ_Add_LayerNorm_Q, LayerNormQ, W8A8BFP32OFP32_GeLu_Q
 from .linear import W8A8B8O8Linear, W8A8B32O32LinearWithoutScaling, W8A8BFP32OFP32Linear
 
@@ -121,7 +121,15 @@ class W8A8OPTDecoderLayer(torch.nn.Module):
         h8 = self.ln1(hidden)
         mark("ln1_layernorm_q")
         w3, b3, a3, s3 = self._qkv_pack()
-        qkv = linear_group_a8_w8_b8_o8(h8, w3, b3, a3, s3, 3)                       # [B,S,3H] int8
+        qkv = None
+        if kv_cache is not None and B == 1 and S <= 16:
+            # decode: projections and KV-cache append in one launch
+            qkv = linear_qkv_decode_a8_w8_b8_o8(h8.view(S, H), w3, b3, a3, s3, kv_cache[0], kv_cache[1])
+        appended = qkv is not None
+        if appended:
+            qkv = qkv.view(1, S, 3 * H)
+        else:
+            qkv = linear_group_a8_w8_b8_o8(h8, w3, b3, a3, s3, 3)                   # [B,S,3H] int8
         q = self._heads(qkv[..., :H], B, S)
         k_new = self._heads(qkv[..., H:2 * H], B, S)
         v = qkv[..., 2 * H:]                                                       # [B,S,H] int8, row pitch 3H
@@ -135,7 +143,9 @@ class W8A8OPTDecoderLayer(torch.nn.Module):
         else:
             # the new K rows and V^T columns go into the last S slots of the cache, one launch per batch
             k_all, vt_all = kv_cache
-            if k_all.is_contiguous() and vt_all.is_contiguous() and self.head_dim % 16 == 0:
+            if appended:
+                pass
+            elif k_all.is_contiguous() and vt_all.is_contiguous() and self.head_dim % 16 == 0:
                 for b in range(B):
                     hs = slice(b * self.heads, (b + 1) * self.heads)
                     kv_append_i8(qkv[b, :, H:2 * H], v[b], k_all[hs], vt_all[hs])
