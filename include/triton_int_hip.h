@@ -174,13 +174,15 @@ int ti_layernorm_q(const float* x, int64_t x_row_stride,
  * resid_out = resid_in + in_scale * f(acc_i32);  y_i8 = q8(LayerNorm(resid_out; gamma, beta, eps)).
  * The native op the reference intends at functional/fused.py:27-32 (module
  * DQ_Add_LayerNorm_Q, nn/fused.py:59-78) and defines only as the PyTorch emulation
- * functional/fused.py:6-15.  in_scale is a host float (nn/fused.py:62,73).  All row-major
+ * functional/fused.py:6-15.  in_scale is a host float (nn/fused.py:62,73); when in_scale_dev is not
+ * NULL the scale is read from that DEVICE fp32 instead and in_scale is ignored (a caller that holds
+ * the scale as a device tensor need not synchronise to fetch it).  All row-major
  * with unit column stride; row strides in elements.  resid_out may alias resid_in.
  * ln_out_f32 (may be NULL) additionally receives the fp32 LayerNorm output, which is what
  * the un-quantised variant returns (functional/fused.py:18-24, dq_add_layernorm); y may be
  * NULL when only that variant is wanted.  At least one of y / ln_out_f32 must be given.
  */
-int ti_dq_add_layernorm_q(const int32_t* acc, int64_t acc_row_stride, float in_scale,
+int ti_dq_add_layernorm_q(const int32_t* acc, int64_t acc_row_stride, float in_scale, const float* in_scale_dev,
                           const float* resid_in, int64_t resid_in_row_stride,
                           const float* gamma, const float* beta, float eps,
                           float* resid_out, int64_t resid_out_row_stride,

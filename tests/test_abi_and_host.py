@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     missing = [n for n in names if not hasattr(lib, n)]
     assert not missing, missing
     assert set(names) == set(_lib.EXPORTS)
-    assert _lib.lib().ti_version() == 1
+    assert _lib.lib().ti_version() == 2
     n = _lib.lib().ti_gemm_num_configs()
     assert n >= 5 and _lib.lib().ti_gemm_config_name(0).decode().startswith("gather")
 
@@ -132,3 +132,83 @@ def test_torch_ops_are_registered_with_meta_implementations():
     o, so = ops.skip_layer_norm_fwd_fused_single_pass2(m((4, 8), torch.float32), m((4, 8), torch.float32), m(8, torch.float32),
                                                        m(8, torch.float32), 1e-5, True)
     assert o.shape == so.shape == (4, 8) and so.dtype == torch.float32
+
+
+def test_reference_import_paths_resolve_to_this_package():
+    """Code written against the reference imports triton_int.* (nn/linear.py:18, nn/bmm.py:10,
+    functional/bmm.py:6); those paths are this package's modules, not copies."""
+    import importlib
+
+    import triton_int
+    import triton_int_amd
+    from triton_int.functional.bmm import bmm_i8_o8, bmm_i8_o32
+    from triton_int.functional.fused import dq_add_layernorm_q_py
+    from triton_int.kernels.bmm import bmm_s8t_s8n_f32t, bmm_s8t_s8n_s8t
+    from triton_int.kernels.fused import layer_norm_fwd_fused_single_pass_q, linear_a8_w8_bfp32_ofp32_GeLu_Q
+    from triton_int.kernels.linear import linear_a8_w8_b8_o8, linear_a8_w8_bfp32_ofp32
+    from triton_int.nn.bmm import BMM_S8T_S8N_F32T, BMM_S8T_S8N_S8T
+    from triton_int.nn.fused import DQ_Add_LayerNorm_Q, LayerNormQ, W8A8BFP32OFP32_GeLu_Q
+    from triton_int.nn.linear import W8A8B8O8Linear, W8A8B8O8LinearReLU, W8A8BFP32OFP32Linear
+
+    assert W8A8B8O8Linear is triton_int_amd.nn.linear.W8A8B8O8Linear
+    assert BMM_S8T_S8N_S8T is triton_int_amd.nn.bmm.BMM_S8T_S8N_S8T
+    assert LayerNormQ is triton_int_amd.nn.fused.LayerNormQ
+    assert linear_a8_w8_b8_o8 is triton_int_amd.kernels.linear.linear_a8_w8_b8_o8
+    assert bmm_i8_o8 is triton_int_amd.functional.bmm.bmm_i8_o8
+    for rel in triton_int.ALIASES:
+        assert importlib.import_module("triton_int." + rel) is importlib.import_module("triton_int_amd." + rel)
+    assert triton_int.nn.linear is triton_int_amd.nn.linear
+    for f in (bmm_i8_o32, dq_add_layernorm_q_py, bmm_s8t_s8n_f32t, bmm_s8t_s8n_s8t, layer_norm_fwd_fused_single_pass_q,
+              linear_a8_w8_bfp32_ofp32_GeLu_Q, linear_a8_w8_bfp32_ofp32, BMM_S8T_S8N_F32T, DQ_Add_LayerNorm_Q,
+              W8A8BFP32OFP32_GeLu_Q, W8A8B8O8LinearReLU, W8A8BFP32OFP32Linear):
+        assert callable(f)
+
+
+def test_c_abi_status_codes_with_raw_ctypes():
+    """Argument errors come back as TI_E_* codes with a message in ti_last_error(), straight from the
+    C ABI (no Python launcher in between).  Argument validation precedes any device access, so no
+    kernel is launched and no GPU is needed."""
+    from triton_int_amd import _lib as L
+    lib = L.lib()
+    TI_E_NULL, TI_E_SHAPE, TI_E_COMBO, TI_E_STRIDE = -1, -2, -3, -4
+    P = 0x1000  # a non-NULL pointer value; never dereferenced on these paths
+
+    def bmm(A=P, B=P, C=P, sC=(0, 64, 1), batch=1, M=32, N=64, K=64, bias=0, bias_kind=L.BIAS_NONE, alpha=P, beta=0,
+            epi=L.EPI_SCALE_I8, dt=L.DT_I8, rnd=L.ROUND_RNE_CLAMP):
+        return lib.ti_bmm_i8(A, 0, K, 1, B, 0, K, 1, C, sC[0], sC[1], sC[2], batch, M, N, K, bias, bias_kind, alpha, beta,
+                             epi, dt, rnd, None)
+
+    def err():
+        return lib.ti_last_error().decode()
+
+    assert bmm(A=0) == TI_E_NULL and "A is NULL" in err()
+    assert bmm(B=0) == TI_E_NULL and "B is NULL" in err()
+    assert bmm(C=0) == TI_E_NULL and "C is NULL" in err()
+    assert bmm(alpha=0) == TI_E_NULL and "alpha" in err()
+    assert bmm(bias=P, bias_kind=L.BIAS_I8, beta=0) == TI_E_NULL and "beta" in err()
+    assert bmm(epi=L.EPI_GELU_I8, beta=0) == TI_E_NULL and "beta" in err()
+    assert bmm(M=-1) == TI_E_SHAPE and "negative" in err()
+    assert bmm(batch=70000) == TI_E_SHAPE and "batch" in err()
+    assert bmm(dt=L.DT_F32) == TI_E_COMBO and "combination" in err()                       # int8 epilogue, fp32 output
+    assert bmm(epi=L.EPI_SCALE_F, dt=L.DT_I8) == TI_E_COMBO
+    assert bmm(bias=P, bias_kind=L.BIAS_F32, beta=P) == TI_E_COMBO                         # fp32 bias on the int8-bias epilogue
+    assert bmm(epi=L.EPI_I32, dt=L.DT_I32, bias=P, bias_kind=L.BIAS_I8) == TI_E_COMBO
+    assert bmm(epi=17) == TI_E_COMBO
+    assert bmm(rnd=5) == TI_E_COMBO and "round mode" in err()
+    assert bmm(sC=(0, 0, 1)) == TI_E_STRIDE and "row stride" in err()
+    assert bmm(sC=(0, 64, 0)) == TI_E_STRIDE and "column stride" in err()
+    # empty problems are no-ops whatever the pointers are
+    assert bmm(A=0, B=0, C=0, M=0) == 0 and bmm(A=0, B=0, C=0, batch=0) == 0
+    # grouped form: negative batch strides of bias / scales
+    assert lib.ti_bmm_i8_grouped(P, 0, 64, 1, P, 0, 64, 1, P, 0, 64, 1, 1, 32, 64, 64, 0, L.BIAS_NONE, -1, P, 0, 0,
+                                 L.EPI_SCALE_I8, L.DT_I8, 0, -1, None) == TI_E_STRIDE
+    # row kernels
+    assert lib.ti_layernorm_q(0, 8, P, P, 1e-5, P, 8, 4, 8, 0, 0, 0, 0, None) == TI_E_NULL
+    assert lib.ti_layernorm_q(P, 8, P, P, 1e-5, P, 8, -4, 8, 0, 0, 0, 0, None) == TI_E_SHAPE
+    assert lib.ti_layernorm_q(P, 8, P, P, 1e-5, P, 8, 4, 8, 0, 9, 0, 0, None) == TI_E_COMBO
+    assert lib.ti_dq_add_layernorm_q(P, 8, 1.0, 0, P, 8, P, P, 1e-5, P, 8, 0, 8, 0, 8, 4, 8, 0, 0, 0, None) == TI_E_NULL  # neither y nor ln_out
+    assert "y / ln_out_f32" in err()
+    assert lib.ti_softmax_q(P, 16, 0.1, P, 16, 4, 16, 32, None) == TI_E_SHAPE               # causal_q_len > cols
+    assert lib.ti_softmax_q(0, 16, 0.1, P, 16, 4, 16, 0, None) == TI_E_NULL
+    assert lib.ti_qkv_decode_i8(P, 64, P, 64, 0, P, P, P, 64, 32, 64, 2048, P, 64, P, 64, 16, None) == TI_E_COMBO  # M > 16
+    assert lib.ti_mfma_i8_probe(-1, 0, None, None) == TI_E_SHAPE

@@ -154,6 +154,27 @@ def test_all_configs_gelu_q(shape):
         assert mx <= 1 and rate < 1e-3, f"{name}: max {mx} rate {rate}"
 
 
+def test_scales_given_as_fp16_fp64_or_host_tensors():
+    """The launchers convert a scale tensor that is not fp32 on the device; both converted copies
+    must be alive at the launch (alpha != beta shows a copy that was freed and re-used)."""
+    linear, bmm, _ = _kl()
+    g = rng(77)
+    a, w, bias = rand_i8(g, 96, 256), rand_i8(g, 80, 256), rand_i8(g, 80)
+    ga, gw, gb = gpu(a), gpu(w), gpu(bias)
+    for alpha, beta in [(0.00390625, 0.25), (0.001953125, 0.75)]:  # exact in fp16
+        want = O.linear_a8_w8_b8_o8(a, w, bias, alpha, beta)
+        for mk in (lambda v: torch.tensor(v, dtype=torch.float16, device=DEV),
+                   lambda v: torch.tensor(v, dtype=torch.float64, device=DEV),
+                   lambda v: torch.tensor(v, dtype=torch.float32),          # host tensor
+                   lambda v: torch.tensor([v], dtype=torch.bfloat16, device=DEV)):
+            got = cpu(linear.linear_a8_w8_b8_o8(ga, gw, gb, mk(alpha), mk(beta)))
+            assert np.array_equal(got, want)
+    bf = g.standard_normal(80).astype(np.float32)
+    got = cpu(linear.linear_a8_w8_bfp32_ofp32(ga, gw, gpu(bf), torch.tensor(0.001953125, dtype=torch.float16, device=DEV),
+                                              torch.tensor(0.75, dtype=torch.float64, device=DEV)))
+    np.testing.assert_array_equal(got, O.linear_a8_w8_bfp32_ofp32(a, w, bf, 0.001953125, 0.75))
+
+
 def test_extreme_accumulators_over_2p24():
     linear, _, _ = _kl()
     K = 2048

@@ -206,3 +206,34 @@ def _clone_linear(lin):
     c = torch.nn.Linear(lin.in_features, lin.out_features)
     c.load_state_dict(lin.state_dict())
     return c
+
+
+def test_reference_usage_through_the_triton_int_import_path():
+    """A caller written against the reference runs unchanged: the imports, constructor, buffer
+    assignment, `.to()` and forward of triton_int/nn/linear.py:18-54 and triton_int/nn/bmm.py:10-29,
+    checked against the oracle."""
+    from triton_int.nn.bmm import BMM_S8T_S8N_S8T
+    from triton_int.nn.linear import W8A8B8O8Linear, W8A8BFP32OFP32Linear
+    from triton_int.kernels.linear import linear_a8_w8_b8_o8
+    from triton_int.functional.bmm import bmm_i8_o8
+    g = rng(21)
+    x = rand_i8(g, 4, 40, 256)
+    w, b = rand_i8(g, 192, 256), rand_i8(g, 192)
+    m = W8A8B8O8Linear(256, 192, alpha=0.0021, beta=0.013)
+    m.weight, m.bias = torch.from_numpy(w), torch.from_numpy(b)
+    m = m.to(DEV)
+    y = m(gpu(x))
+    want = O.linear_a8_w8_b8_o8(x.reshape(-1, 256), w, b, 0.0021, 0.013).reshape(4, 40, 192)
+    assert y.shape == (4, 40, 192) and np.array_equal(cpu(y), want)
+    assert np.array_equal(cpu(linear_a8_w8_b8_o8(gpu(x), gpu(w), gpu(b), m.a, m.b)), want)
+    bf = g.standard_normal(192).astype(np.float32)
+    m2 = W8A8BFP32OFP32Linear(256, 192, alpha=0.003)
+    m2.weight, m2.bias = torch.from_numpy(w), torch.from_numpy(bf)
+    m2 = m2.to(DEV)
+    np.testing.assert_array_equal(cpu(m2(gpu(x))),
+                                  O.linear_a8_w8_bfp32_ofp32(x.reshape(-1, 256), w, bf, 0.003, 1.0).reshape(4, 40, 192))
+    q, k = rand_i8(g, 6, 48, 64), rand_i8(g, 6, 80, 64)
+    bmm = BMM_S8T_S8N_S8T(1e-3).to(DEV)
+    want_s = O.bmm_s8t_s8n_s8t(q, k, np.float32(1e-3))
+    assert np.array_equal(cpu(bmm(gpu(q), gpu(k))), want_s)
+    assert np.array_equal(cpu(bmm_i8_o8(gpu(q), gpu(k), 1e-3)), want_s)

@@ -122,6 +122,12 @@ def test_dq_add_layernorm_q_shapes(rows, cols):
     assert np.array_equal(cpu(rout), o_rout)
     mx, rate = mismatch_report(cpu(q), o_q)
     assert mx <= 1 and rate <= max(INT8_MISMATCH_RATE, 1.5 / o_q.size)
+    # the scale as a device tensor is read by the kernel (no host synchronisation): same bits
+    s_dev = torch.tensor(3e-5, dtype=torch.float32, device=DEV)
+    rout2, q2 = fused.dq_add_layernorm_q(gpu(acc), s_dev, gpu(res), gpu(w), gpu(b), 1e-5)
+    assert torch.equal(rout2, rout) and torch.equal(q2, q)
+    rout3, q3 = fused.dq_add_layernorm_q(gpu(acc), torch.tensor(3e-5, dtype=torch.float64), gpu(res), gpu(w), gpu(b), 1e-5)
+    assert torch.equal(rout3, rout) and torch.equal(q3, q)
 
 
 @pytest.mark.parametrize("n", [1, 3, 4, 1000, 4099, 2048 * 16384])

@@ -59,7 +59,7 @@ def _declare(lib):
     lib.ti_layernorm_q.restype = _int
     lib.ti_layernorm_q.argtypes = [_vp, _i64, _vp, _vp, _f32, _vp, _i64, _int, _int, _int, _int, _vp, _vp, _vp]
     lib.ti_dq_add_layernorm_q.restype = _int
-    lib.ti_dq_add_layernorm_q.argtypes = [_vp, _i64, _f32, _vp, _i64, _vp, _vp, _f32, _vp, _i64, _vp, _i64,
+    lib.ti_dq_add_layernorm_q.argtypes = [_vp, _i64, _f32, _vp, _vp, _i64, _vp, _vp, _f32, _vp, _i64, _vp, _i64,
                                           _vp, _i64, _int, _int, _int, _vp, _vp, _vp]
     lib.ti_softmax_q.restype = _int
     lib.ti_softmax_q.argtypes = [_vp, _i64, _f32, _vp, _i64, _int, _int, _int, _vp]
@@ -160,8 +160,14 @@ def scale_tensor(v, device) -> torch.Tensor:
     key = (float(v), str(device))
     t = _scalar_cache.get(key)
     if t is None:
-        if len(_scalar_cache) > 4096:
-            _scalar_cache.clear()
+        # Entries are never evicted: a captured HIP graph keeps the device address of every scale it
+        # was recorded with (4 bytes per distinct value and device).  The upload is a synchronous
+        # host-to-device copy, which a capturing stream cannot record: pass the scale as a device
+        # tensor, or call once with the same value before the capture.
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError(
+                f"scale {float(v)!r} was first seen during HIP graph capture; pass scales as fp32 device "
+                "tensors, or run the call once before capturing")
         t = torch.tensor(float(v), dtype=torch.float32, device=device)
         _scalar_cache[key] = t
     return t

@@ -52,10 +52,6 @@ struct GemmParams {
 
 enum OutClass { OUT8 = 0, OUT32 = 1, OUT16 = 2 };
 
-#ifdef TI_TRACE
-// debug builds only: per-wave cycle counts of the main loop (never compiled into the product)
-__device__ unsigned long long ti_trace_buf[8192];
-#endif
 
 // ---- tile -> (m, n) mapping ----------------------------------------------------------------
 // Workgroups are dealt round-robin to the 8 XCDs (each with a private L2), so consecutive
@@ -923,10 +919,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
       for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-#ifdef TI_TRACE
-    const uint64_t tr_a = wall_clock64();
-    const uint64_t tr_ca = __builtin_readcyclecounter();
-#endif
     // k-tile 0 of this item has landed: the barrier of the previous k-tile (or the one above) saw to it
 #pragma unroll
     for (int r = 0; r < NR; ++r) load_frag(lds + st * STAGE, 0, 0, r);
@@ -949,19 +941,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
       dma_advance();
     }
 
-#ifdef TI_TRACE
-    const uint64_t tr_b = wall_clock64();
-    const uint64_t tr_cb = __builtin_readcyclecounter();
-#endif
     // ---- epilogue
     stream_epilogue<TM, TN, OUTCLS>(p, e, acc, bz, m0 + wm * WTM, n0 + wn * WTN,
                                     lds + NSTAGE * STAGE + wave * (STRIP + COLS), lane);
-#ifdef TI_TRACE
-    if (lane == 0 && blockIdx.x < 256 && it == 2) {
-      unsigned long long* tr = ti_trace_buf + (blockIdx.x * 4 + (wave & 3)) * 8;
-      tr[0] = tr_a; tr[1] = tr_b; tr[2] = wall_clock64(); tr[3] = tr_cb - tr_ca; tr[4] = __builtin_readcyclecounter() - tr_cb;
-    }
-#endif
   }
   // the trailing (empty-buffer) loads still write zeros into LDS: they must land before the
   // workgroup's LDS is handed to another one
@@ -1103,29 +1085,10 @@ __global__ __launch_bounds__((WAVES_M * WAVES_N + PW) * 64) void gemm_mfma_ws_ke
     for (int t = 0; t < DEPTH; ++t) issue_ktile();
     wait_loads_and_barrier<LOADS*(DEPTH - 1)>();  // k-tile 0 landed
     const int total = count * KT;
-#ifdef TI_TRACE
-    uint64_t tr_issue = 0, tr_wait = 0, tr_bar = 0;
-    const uint64_t tr_w0 = wall_clock64();
-    for (int g = 0; g < total; ++g) {
-      const uint64_t c0 = __builtin_readcyclecounter();
-      issue_ktile();
-      const uint64_t c1 = __builtin_readcyclecounter();
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS*(DEPTH - 1)) : "memory");
-      const uint64_t c2 = __builtin_readcyclecounter();
-      asm volatile("s_barrier" ::: "memory");
-      const uint64_t c3 = __builtin_readcyclecounter();
-      tr_issue += c1 - c0; tr_wait += c2 - c1; tr_bar += c3 - c2;
-    }
-    if (lane == 0 && blockIdx.x < 256) {
-      unsigned long long* tr = ti_trace_buf + (blockIdx.x * 4 + (wave & 3)) * 8;
-      tr[0] = tr_issue; tr[1] = tr_wait; tr[2] = tr_bar; tr[3] = total; tr[4] = wall_clock64() - tr_w0;
-    }
-#else
     for (int g = 0; g < total; ++g) {
       issue_ktile();                                // k-tile g + DEPTH
       wait_loads_and_barrier<LOADS*(DEPTH - 1)>();  // k-tile g + 1 landed; barrier g
     }
-#endif
     // the trailing (empty-buffer) loads still write zeros into LDS: they must land before the
     // workgroup's LDS is handed to another one
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -1276,9 +1239,6 @@ __global__ __launch_bounds__(512, UU ? 2 : 4) void gemm_skinny_kernel(GemmParams
   constexpr int U = UU ? UU : (MBMAX * G == 1 ? 6 : 8 / (MBMAX * G));  // k-steps per batch of loads; two batches are in flight
   __shared__ int red[NW][G * MBMAX][256];
   const int tid = threadIdx.x, lane = tid & 63;
-#ifdef TI_TRACE
-  const uint64_t tr0 = wall_clock64();
-#endif
   // The wave index must be known to be wave-uniform: the trip counts below depend on it, and a
   // branch the compiler believes divergent would wrap MFMAs in EXEC masking, which MFMAs ignore.
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1389,9 +1349,6 @@ __global__ __launch_bounds__(512, UU ? 2 : 4) void gemm_skinny_kernel(GemmParams
     }
   }
 
-#ifdef TI_TRACE
-  const uint64_t tr1 = wall_clock64();
-#endif
   if (ksplit > 1) {
 #pragma unroll
     for (int g = 0; g < G; ++g)
@@ -1408,9 +1365,6 @@ __global__ __launch_bounds__(512, UU ? 2 : 4) void gemm_skinny_kernel(GemmParams
           for (int kp = 1; kp < ksplit; ++kp) acc[g][mb] += *(const v4i*)&red[wave + kp][g * MBMAX + mb][lane * 4];
   }
 
-#ifdef TI_TRACE
-  const uint64_t tr2 = wall_clock64();
-#endif
   // acc[g][mb][i]: n = (group*G + g)*16 + 4*c4 + i, m = mb*16 + r16
   constexpr int ESZ = OUTCLS == OUT8 ? 1 : (OUTCLS == OUT32 ? 4 : 2);
   char* Cz = (char*)p.C + (int64_t)bz * p.sCb * ESZ;
@@ -1429,12 +1383,6 @@ __global__ __launch_bounds__(512, UU ? 2 : 4) void gemm_skinny_kernel(GemmParams
       }
     }
   }
-#ifdef TI_TRACE
-  if (lane == 0 && blockIdx.x < 1024 && kpart == 0 && (wave / ksplit) == 0) {
-    unsigned long long* tr = ti_trace_buf + blockIdx.x * 8;
-    tr[0] = tr0; tr[1] = tr1; tr[2] = tr2; tr[3] = wall_clock64();
-  }
-#endif
 }
 
 // ---- decode kernel: M <= 16, weights streamed as whole 1 KB row pieces ----------------------------
@@ -2088,11 +2036,6 @@ int ti_linear_i8_residual_f32(const int8_t* A, int64_t lda, const int8_t* W, int
   return ti::run_with_residual(p, residual, ldr, (hipStream_t)stream);
 }
 
-#ifdef TI_TRACE
-int ti_debug_trace(unsigned long long* dst, int n) {
-  return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(ti::ti_trace_buf), sizeof(unsigned long long) * n);
-}
-#endif
 
 int ti_gemm_num_configs(void) { return ti::g_num_configs; }
 

@@ -96,7 +96,7 @@ __global__ __launch_bounds__(PROBE_THREADS) void mfma_probe_kernel(int iters, in
 
 extern "C" {
 
-int ti_version(void) { return 1; }
+int ti_version(void) { return 2; }
 
 int ti_mfma_i8_probe(int iters, int random_operands, void* stream, double* ops_out) {
   if (iters < 0) return ti::fail(TI_E_SHAPE, "negative iteration count");

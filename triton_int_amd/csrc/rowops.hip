@@ -42,6 +42,7 @@ struct RowNormParams {
   float* resid_out;      // DQ
   int64_t x_rs, acc_rs, rin_rs, rout_rs, y_rs, ln_rs;
   float in_scale;
+  const float* in_scale_dev;  // when given, the dequantisation scale is read from device memory
   const float* gamma;
   const float* beta;
   float eps;
@@ -94,6 +95,10 @@ __global__ __launch_bounds__(RN_THREADS) void rownorm_vec_kernel(RowNormParams p
   }
   const float inv_n = 1.0f / (float)p.cols;
   const bool y_vec = p.y && ((p.y_rs & 3) == 0) && ((((uintptr_t)p.y) & 3) == 0);
+  float in_scale = p.in_scale;
+  if constexpr (DQ) {
+    if (p.in_scale_dev) in_scale = *p.in_scale_dev;
+  }
 
   for (; row < p.rows; row += gridDim.x) {
     if constexpr (DQ) {
@@ -107,7 +112,7 @@ __global__ __launch_bounds__(RN_THREADS) void rownorm_vec_kernel(RowNormParams p
 #pragma unroll
           for (int t = 0; t < 4; ++t) {
             // functional/fused.py:9: residual + alpha * int32 (product and sum rounded separately)
-            const float prod = p.in_scale * (float)a[t];
+            const float prod = in_scale * (float)a[t];
             o[t] = r[t] + prod;
           }
           x[j] = o;
@@ -180,8 +185,9 @@ __global__ __launch_bounds__(RN_THREADS) void rownorm_any_kernel(RowNormParams p
     const int32_t* ar = p.acc + (int64_t)row * p.acc_rs;
     const float* rin = p.resid_in + (int64_t)row * p.rin_rs;
     float* rout = p.resid_out + (int64_t)row * p.rout_rs;
+    const float in_scale = p.in_scale_dev ? *p.in_scale_dev : p.in_scale;
     for (int i = tid; i < p.cols; i += RN_THREADS) {
-      const float prod = p.in_scale * (float)ar[i];
+      const float prod = in_scale * (float)ar[i];
       rout[i] = rin[i] + prod;
     }
     __threadfence_block();
@@ -598,8 +604,8 @@ int ti_layernorm_q(const float* x, int64_t x_row_stride, const float* gamma, con
   return ti::launch_rownorm<false>(p, (hipStream_t)stream);
 }
 
-int ti_dq_add_layernorm_q(const int32_t* acc, int64_t acc_row_stride, float in_scale, const float* resid_in,
-                          int64_t resid_in_row_stride, const float* gamma, const float* beta, float eps,
+int ti_dq_add_layernorm_q(const int32_t* acc, int64_t acc_row_stride, float in_scale, const float* in_scale_dev,
+                          const float* resid_in, int64_t resid_in_row_stride, const float* gamma, const float* beta, float eps,
                           float* resid_out, int64_t resid_out_row_stride, int8_t* y, int64_t y_row_stride,
                           float* ln_out_f32, int64_t ln_out_row_stride, int rows, int cols, int round_mode,
                           float* mean_out, float* rstd_out, void* stream) {
@@ -609,7 +615,7 @@ int ti_dq_add_layernorm_q(const int32_t* acc, int64_t acc_row_stride, float in_s
   if (!y && !ln_out_f32) return ti::fail(TI_E_NULL, "one of y / ln_out_f32 is required");
   if (round_mode != TI_ROUND_RNE_CLAMP && round_mode != TI_ROUND_TRUNC) return ti::fail(TI_E_COMBO, "round mode %d", round_mode);
   ti::RowNormParams p = {};
-  p.acc = acc; p.acc_rs = acc_row_stride; p.in_scale = in_scale;
+  p.acc = acc; p.acc_rs = acc_row_stride; p.in_scale = in_scale; p.in_scale_dev = in_scale_dev;
   p.resid_in = resid_in; p.rin_rs = resid_in_row_stride;
   p.resid_out = resid_out; p.rout_rs = resid_out_row_stride;
   p.gamma = gamma; p.beta = beta; p.eps = eps;

@@ -37,12 +37,14 @@ def _launch(a, sa, b, sb, c, sc, B, M, N, K, *, epilogue, bias, alpha, beta, rou
         if rc != 0:
             L.check(rc, "ti_bmm_i8_grouped")
         return
-    alpha_ptr = 0 if alpha is None else L.scale_tensor(alpha, dev).data_ptr()
-    beta_ptr = 0 if beta is None else L.scale_tensor(beta, dev).data_ptr()
+    # the converted scales stay bound to locals until the launch is enqueued: a scale that is not
+    # already fp32 on `dev` is a fresh copy, and a freed copy's block would be handed to the next one
+    alpha_t = None if alpha is None else L.scale_tensor(alpha, dev)
+    beta_t = None if beta is None else L.scale_tensor(beta, dev)
     with L.on_device(dev):
         rc = L.lib().ti_bmm_i8_config(
             a.data_ptr(), sa[0], sa[1], sa[2], b.data_ptr(), sb[0], sb[1], sb[2], c.data_ptr(), sc[0], sc[1], sc[2],
-            B, M, N, K, bias_ptr, bias_kind, alpha_ptr, beta_ptr,
+            B, M, N, K, bias_ptr, bias_kind, L.ptr(alpha_t), L.ptr(beta_t),
             int(epilogue), L.TORCH_TO_DT[c.dtype], int(round_mode), int(config), L.current_stream(dev))
     if rc != 0:
         L.check(rc, "ti_bmm_i8")

@@ -133,11 +133,19 @@ def dq_add_layernorm_q(input_int32, input_scale_fp, residual_input_fp, gamma, be
     if _return_stats:
         mean = torch.empty(rows, dtype=torch.float32, device=dev)
         rstd = torch.empty(rows, dtype=torch.float32, device=dev)
+    # the module holds a python float (nn/fused.py:62); a tensor scale is read on the device, so that
+    # the call neither synchronises nor breaks a graph capture
+    scale_t = None
     if torch.is_tensor(input_scale_fp):
-        input_scale_fp = float(input_scale_fp)  # the module holds a python float (nn/fused.py:62)
+        scale_t = input_scale_fp if input_scale_fp.is_cuda else None
+        if scale_t is None:
+            input_scale_fp = float(input_scale_fp)
+        else:
+            scale_t = L.scale_tensor(scale_t.reshape(()), dev)
+            input_scale_fp = 0.0
     with L.on_device(dev):
         rc = L.lib().ti_dq_add_layernorm_q(
-            L.ptr(acc), acc.stride(0) if rows > 1 else H, float(input_scale_fp), L.ptr(rin),
+            L.ptr(acc), acc.stride(0) if rows > 1 else H, float(input_scale_fp), L.ptr(scale_t), L.ptr(rin),
             rin.stride(0) if rows > 1 else H, L.ptr(gamma), L.ptr(beta), float(eps), L.ptr(rout), H, L.ptr(y), H,
             L.ptr(ln), H, rows, H, int(_round_mode), L.ptr(mean), L.ptr(rstd), L.current_stream(dev))
     L.check(rc, "ti_dq_add_layernorm_q")
