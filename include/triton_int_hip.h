@@ -118,8 +118,13 @@ int ti_bmm_i8(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk,
  * Same as ti_bmm_i8 but forces one kernel configuration (index into the library's tile
  * table; see ti_gemm_num_configs / ti_gemm_config_name).  Used by the tuner and the
  * parity tests so that every configuration is checked, not only the one the dispatcher
- * would pick.  config = -1 selects automatically.  Returns TI_E_COMBO if the
- * configuration cannot run the given stride pattern.
+ * would pick.  config = -1 selects automatically.  Bits 8..15 of a non-negative config force
+ * the number of K splits of a wave-specialised ("ws_") configuration (0 = choose; bits 0..7 equal
+ * to 0xff = choose the configuration): K is dealt to that many work items per tile, whose int32
+ * partial sums meet in a workspace the library keeps per device and stream (allocated on first
+ * use, up to 96 MiB; never during a graph capture, where an unsplit launch is used if there is
+ * none yet).  Integer sums: the result does not depend on the split.  Returns TI_E_COMBO if the
+ * configuration cannot run the given stride pattern or cannot split K.
  */
 int ti_bmm_i8_config(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk,
                      const int8_t* B, int64_t sBb, int64_t sBn, int64_t sBk,
@@ -152,6 +157,8 @@ const char* ti_gemm_config_name(int config);
 /* Index of the configuration the calling thread's most recent ti_bmm_i8* launch used (-1 if
  * none); lets a benchmark attribute time to the kernel that actually ran. */
 int ti_gemm_last_config(void);
+/* Number of K splits that launch used (1 = K not split). */
+int ti_gemm_last_splits(void);
 
 /* ---- row kernels ------------------------------------------------------------------- */
 

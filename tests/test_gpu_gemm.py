@@ -365,7 +365,8 @@ def test_baseline_config2_opt67b_shapes_sampled_rows(which):
 
 @pytest.mark.parametrize("M,N,K", [(16, 5120, 5120), (1, 5120, 5120), (17, 272, 1040), (48, 100, 64), (64, 20480, 5120), (16, 5120, 20480)])
 def test_decode_shapes_skinny_kernel(M, N, K):
-    """M <= 64 takes the weight-streaming kernel (K split across waves, int32 partials added in LDS)."""
+    """M <= 16 takes a weight-streaming kernel (row pieces, or slabs with K split across waves); up to
+    128 rows against a long K take 128 x 128 tiles with K split over workgroups; short K the slabs."""
     linear, _, fused = _kl()
     L = _lib()
     g = rng(M * 13 + N)
@@ -374,7 +375,8 @@ def test_decode_shapes_skinny_kernel(M, N, K):
     b8 = rand_i8(g, N); bf = g.standard_normal(N).astype(np.float32)
     ga, gw = gpu(a), gpu(w)
     got = cpu(linear.linear_a8_w8_b32_o32(ga, gw, gpu(b32)))
-    assert L.lib().ti_gemm_config_name(L.lib().ti_gemm_last_config()).decode().startswith(("skinny", "rows4"))
+    used = L.lib().ti_gemm_config_name(L.lib().ti_gemm_last_config()).decode()
+    assert used.startswith(("skinny", "rows4") if (M <= 16 or K < 1024) else "ws_128x128"), used
     assert np.array_equal(got, O.linear_a8_w8_b32_o32(a, w, b32))
     alpha = np.float32(40.0 / (np.sqrt(K) * 127 * 127 / 3)); beta = np.float32(0.05)
     assert np.array_equal(cpu(linear.linear_a8_w8_b8_o8(ga, gw, gpu(b8), alpha, beta)), O.linear_a8_w8_b8_o8(a, w, b8, alpha, beta))
@@ -386,6 +388,76 @@ def test_decode_shapes_skinny_kernel(M, N, K):
     mx, rate = mismatch_report(cpu(fused.linear_a8_w8_bfp32_ofp32_GeLu_Q(ga, gw, gpu(bf), ag, 20.0)),
                                O.linear_a8_w8_bfp32_ofp32_GeLu_Q(a, w, bf, ag, np.float32(20.0)))
     assert mx <= 1 and rate < 1e-3
+
+
+@pytest.mark.parametrize("M,N,K", [(130, 272, 2064), (300, 400, 1040), (64, 400, 4096), (33, 112, 2048), (700, 144, 4112)])
+def test_split_k_every_ws_config_bit_exact(M, N, K):
+    """K dealt to 2..8 work items per tile (forced through bits 8..15 of the configuration argument):
+    int32 partial sums meet in the library's workspace, the last item of a tile stores it.  Integer
+    sums, so every split count must give the oracle's bits, twice in a row (the ticket counters must
+    be back at zero after a launch), for ragged M / N, a K tail and more splits than k-tiles."""
+    linear, _, fused = _kl()
+    L = _lib()
+    g = rng(M + 3 * N + K)
+    a, w = rand_i8(g, M, K, lo=-128), rand_i8(g, N, K, lo=-128)
+    b32 = g.integers(-2**20, 2**20, size=N, dtype=np.int32)
+    b8 = rand_i8(g, N); bf = g.standard_normal(N).astype(np.float32)
+    ga, gw, gb32, gb8, gbf = gpu(a), gpu(w), gpu(b32), gpu(b8), gpu(bf)
+    alpha = np.float32(40.0 / (np.sqrt(K) * 127 * 127 / 3)); beta = np.float32(0.05)
+    want32 = O.linear_a8_w8_b32_o32(a, w, b32)
+    want8 = O.linear_a8_w8_b8_o8(a, w, b8, alpha, beta)
+    wantf = O.linear_a8_w8_bfp32_ofp32(a, w, bf, alpha, 1.0)
+    ran = 0
+    for cfg, name in _configs(M, N, out8=True):
+        if not name.startswith("ws_"):
+            continue
+        for splits in (2, 3, 5, 8, 40):
+            forced = cfg | (splits << 8)
+            for _ in range(2):
+                assert np.array_equal(cpu(linear.linear_a8_w8_b32_o32(ga, gw, gb32, _config=forced)), want32), (name, splits)
+                used = L.lib().ti_gemm_last_splits()
+                assert 1 < used <= min(splits, (K + 127) // 128), (name, splits, used)
+                assert np.array_equal(cpu(linear.linear_a8_w8_b8_o8(ga, gw, gb8, alpha, beta, _config=forced)), want8), (name, splits)
+                assert np.array_equal(cpu(linear.linear_a8_w8_bfp32_ofp32(ga, gw, gbf, alpha, 1.0, _config=forced)), wantf), (name, splits)
+            ran += 1
+    assert ran >= 15
+    # a configuration that cannot split refuses a forced split; the automatic choice never fails
+    with pytest.raises(AssertionError, match="cannot split K"):
+        linear.linear_a8_w8_b32_o32(ga, gw, gb32, _config=1 | (2 << 8))
+    assert np.array_equal(cpu(linear.linear_a8_w8_b32_o32(ga, gw, gb32)), want32)
+
+
+def test_split_k_on_two_streams_and_under_graph_capture():
+    """Launches on different streams get their own workspace (they may overlap); a launch captured into
+    a graph uses the workspace its stream already has and replays correctly."""
+    linear, _, _ = _kl()
+    L = _lib()
+    g = rng(5)
+    M, N, K = 128, 1024, 4096
+    a, w, b32 = rand_i8(g, M, K), rand_i8(g, N, K), g.integers(-2**20, 2**20, size=N, dtype=np.int32)
+    ga, gw, gb = gpu(a), gpu(w), gpu(b32)
+    want = O.linear_a8_w8_b32_o32(a, w, b32)
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    outs = []
+    torch.cuda.synchronize()
+    for _ in range(4):
+        for st in (s1, s2):
+            with torch.cuda.stream(st):
+                outs.append(linear.linear_a8_w8_b32_o32(ga, gw, gb))
+                assert L.lib().ti_gemm_last_splits() > 1
+    torch.cuda.synchronize()
+    for o in outs:
+        assert np.array_equal(cpu(o), want)
+    out = torch.empty((M, N), dtype=torch.int32, device=DEV)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(s1):
+        with torch.cuda.graph(graph, stream=s1):
+            linear.linear_a8_w8_b32_o32(ga, gw, gb, out=out)
+    for _ in range(3):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(cpu(out), want)
 
 
 @pytest.mark.parametrize("M,N,K", [(16, 5136, 1104), (9, 400, 2048), (1, 48, 64), (13, 5120, 5120)])

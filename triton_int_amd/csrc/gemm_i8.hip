@@ -16,7 +16,9 @@
 //
 // C = epilogue(sum_k A[m,k] * B[n,k]); A is [M,K], B is [N,K] (the reference's "N" operand,
 // kernels/linear.py:217), the "T" operand [K,N] arrives as strides (sBn = 1, sBk = N).
+#include <mutex>
 #include <type_traits>
+#include <vector>
 
 #include "ti_common.h"
 
@@ -48,6 +50,12 @@ struct GemmParams {
   int8_t* kv_vt;
   int64_t kv_k_hs, kv_vt_rs;
   int kv_D;
+  // split K (gemm_mfma_ws_kernel, batch == 1): a tile's k-tiles are dealt to `splits` work items of
+  // kt_split k-tiles each (the last takes what is left); the items leave their int32 sums in
+  // sk_partial, and the item of a tile that finishes last adds them up and stores the tile.
+  int splits, kt_split;
+  int* sk_partial;   // [tile][split][consumer wave][accumulator dword][lane]
+  int* sk_counter;   // [tile][consumer wave], zero between launches
 };
 
 enum OutClass { OUT8 = 0, OUT32 = 1, OUT16 = 2 };
@@ -991,9 +999,12 @@ __global__ __launch_bounds__((WAVES_M * WAVES_N + PW) * 64) void gemm_mfma_ws_ke
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-  // ---- this workgroup's items: ranks first, first + step, ... (count of them)
+  // ---- this workgroup's items: ranks first, first + step, ... (count of them).  An item is a tile
+  // of a batch entry, or, with split K (batch == 1), one of the `splits` runs of k-tiles of a tile;
+  // the runs of a tile are neighbours in the list, so they are worked on at the same time.
   const int T = p.tiles_m * p.tiles_n;
-  const int W = T * p.batch;
+  const int SPL = p.splits;
+  const int W = T * p.batch * SPL;
   int first, step, count;
   {
     const int G = (int)gridDim.x, b = (int)blockIdx.x;
@@ -1014,16 +1025,26 @@ __global__ __launch_bounds__((WAVES_M * WAVES_N + PW) * 64) void gemm_mfma_ws_ke
     count = __builtin_amdgcn_readfirstlane(count);
   }
   if (count == 0) return;
-  auto locate = [&](int i, int& bz, int& m0, int& n0) {
-    const int g = first + i * step;
+  const int KT = (p.K + BK - 1) / BK;
+  // item i: batch entry bz, tile origin (m0, n0), tile rank, split s with k-tiles [kt0, kt0 + kts)
+  auto locate = [&](int i, int& bz, int& m0, int& n0, int& rank, int& s, int& kt0, int& kts) {
+    int g = first + i * step;
+    int s_ = 0;
+    if (SPL > 1) {
+      s_ = g % SPL;
+      g /= SPL;
+    }
     const int b_ = g / T;
     int tm, tn;
     tile_from_rank(p, g - b_ * T, tm, tn);
     bz = __builtin_amdgcn_readfirstlane(b_);
     m0 = __builtin_amdgcn_readfirstlane(tm * BM);
     n0 = __builtin_amdgcn_readfirstlane(tn * BN);
+    rank = __builtin_amdgcn_readfirstlane(g - b_ * T);
+    s = __builtin_amdgcn_readfirstlane(s_);
+    kt0 = SPL > 1 ? s * p.kt_split : 0;
+    kts = SPL > 1 ? min(p.kt_split, KT - kt0) : KT;
   };
-  const int KT = (p.K + BK - 1) / BK;
   const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
 
   if (wave >= NWC) {
@@ -1047,8 +1068,10 @@ __global__ __launch_bounds__((WAVES_M * WAVES_N + PW) * 64) void gemm_mfma_ws_ke
       kt_left = KT;
       k_issue = 0;
       if (i < count) {
-        int bz, m0, n0;
-        locate(i, bz, m0, n0);
+        int bz, m0, n0, rank, sp, kt0, kts;
+        locate(i, bz, m0, n0, rank, sp, kt0, kts);
+        kt_left = kts;
+        k_issue = kt0 * BK;
         // rows at or past M (N) and bytes past K of the last row read as zero
         rA = make_rsrc(p.A + (int64_t)bz * p.sAb + (int64_t)m0 * lda, (p.M - 1 - m0) * lda + p.K);
         rB = make_rsrc(p.B + (int64_t)bz * p.sBb + (int64_t)n0 * ldb, (p.N - 1 - n0) * ldb + p.K);
@@ -1084,7 +1107,15 @@ __global__ __launch_bounds__((WAVES_M * WAVES_N + PW) * 64) void gemm_mfma_ws_ke
 #pragma unroll
     for (int t = 0; t < DEPTH; ++t) issue_ktile();
     wait_loads_and_barrier<LOADS*(DEPTH - 1)>();  // k-tile 0 landed
-    const int total = count * KT;
+    int total = count * KT;  // k-tiles of all items = barriers to join
+    if (SPL > 1) {
+      total = 0;
+      for (int i = 0; i < count; ++i) {
+        int bz, m0, n0, rank, sp, kt0, kts;
+        locate(i, bz, m0, n0, rank, sp, kt0, kts);
+        total += kts;
+      }
+    }
     for (int g = 0; g < total; ++g) {
       issue_ktile();                                // k-tile g + DEPTH
       wait_loads_and_barrier<LOADS*(DEPTH - 1)>();  // k-tile g + 1 landed; barrier g
@@ -1117,22 +1148,32 @@ __global__ __launch_bounds__((WAVES_M * WAVES_N + PW) * 64) void gemm_mfma_ws_ke
       acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
   };
   constexpr int NM = TM * TN, NR = TM + TN;
-  // one k-step, pinned order: MFMA u, then fragment read u of the following k-step
-  auto kstep = [&](int buf, const char* rd_stage, int rd_ks) {
+  // One k-step, pinned order: MFMA u, then RPM fragment reads of the following k-step.  The reads go
+  // out in the order in which the next k-step's MFMAs (i major, j minor) first touch a fragment:
+  // A0, B0 .. B(TN-1), A1 .. A(TM-1), so that every fragment has most of a k-step of MFMAs between
+  // its read and its first use (an LDS read takes longer than three MFMAs to come back).
+  auto kstep = [&](int buf, const char* rd_stage, int rd_ks, auto rpm_tag) {
+    constexpr int RPM_ = decltype(rpm_tag)::value;
+    constexpr int RPM = RPM_ * NM >= NR ? RPM_ : (NR + NM - 1) / NM;
 #pragma unroll
     for (int u = 0; u < NM; ++u) {
       mfma(buf, u);
 #pragma unroll
-      for (int r = 0; r < NR; ++r)
-        if (NM > NR ? r == u : r * NM / NR == u) load_frag(rd_stage, rd_ks, buf ^ 1, r);
+      for (int s = u * RPM; s < (u + 1) * RPM; ++s)
+        if (s < NR) {
+          const int r = s == 0 ? 0 : (s <= TN ? TM + s - 1 : s - TN);
+          load_frag(rd_stage, rd_ks, buf ^ 1, r);
+        }
       __builtin_amdgcn_sched_barrier(0);
     }
   };
+  using Rpm1 = std::integral_constant<int, 1>;
+  using RpmLast = std::integral_constant<int, 2>;
   asm volatile("s_barrier" ::: "memory");  // k-tile 0 is in LDS
   int st = 0;
   for (int it = 0; it < count; ++it) {
-    int bz, m0, n0;
-    locate(it, bz, m0, n0);
+    int bz, m0, n0, rank, sp, kt0, kts;
+    locate(it, bz, m0, n0, rank, sp, kt0, kts);
     const EpiCtx e = make_epi(p, bz);  // scalar loads, long done when the epilogue needs them
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -1142,16 +1183,62 @@ __global__ __launch_bounds__((WAVES_M * WAVES_N + PW) * 64) void gemm_mfma_ws_ke
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 #pragma unroll
     for (int r = 0; r < NR; ++r) load_frag(lds + st * STAGE, 0, 0, r);
-    for (int kt = 0; kt < KT; ++kt) {
+    for (int kt = 0; kt < kts; ++kt) {
       const char* cur = lds + st * STAGE;
       st = (st + 1 == NSTAGE) ? 0 : st + 1;
 #pragma unroll
-      for (int ks = 0; ks < KS - 1; ++ks) kstep(ks & 1, cur, ks + 1);
+      for (int ks = 0; ks < KS - 2; ++ks) kstep(ks & 1, cur, ks + 1, Rpm1{});
+      // the k-step before the barrier issues its reads early (two per MFMA), so that they have come
+      // back when the barrier is reached
+      kstep((KS - 2) & 1, cur, KS - 1, RpmLast{});
       // every LDS read of this k-tile is issued: wait for them, then hand the stage back
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
       // last k-step; the fragments it fetches are the first of the next k-tile (of the next item
       // after the last k-tile: landed as well, and simply fetched again at the item's start)
-      kstep((KS - 1) & 1, lds + st * STAGE, 0);
+      kstep((KS - 1) & 1, lds + st * STAGE, 0, Rpm1{});
+    }
+    if (SPL > 1) {
+      // Split K.  Each consumer wave settles its own quarter of the tile with the same wave of the
+      // tile's other items, no workgroup barrier involved: it stores its sums (every instruction
+      // 64 lanes x 16 consecutive bytes), waits until they are written and takes a ticket from the
+      // quarter's counter.  The wave that draws the last ticket knows that all the others' sums are
+      // in memory: it adds them to its own (integer sums: any order gives the same bits), puts the
+      // counter back to zero for the next launch and stores the tile.  Nobody waits for anybody.
+      // The sums travel with device-scope cache policy (sc1: written through to, and read from,
+      // the memory side that all XCDs share), so no cache-wide write-back or invalidation is needed.
+      constexpr int WAVE_BYTES = TM * TN * 16 * 64 * 4;
+      constexpr int SC1 = 16;
+      const __amdgpu_buffer_rsrc_t rP = __builtin_amdgcn_make_buffer_rsrc(p.sk_partial, 0, 0x7ffffff0, 0x00020000);
+      const int mine = ((rank * SPL + sp) * NWC + wave) * WAVE_BYTES + lane * 16;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            __builtin_amdgcn_raw_buffer_store_b128(
+                (v4u){(unsigned)acc[i][j][4 * q], (unsigned)acc[i][j][4 * q + 1], (unsigned)acc[i][j][4 * q + 2], (unsigned)acc[i][j][4 * q + 3]},
+                rP, mine + ((i * TN + j) * 4 + q) * 1024, 0, SC1);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      int ticket = 0;
+      if (lane == 0) ticket = atomicAdd(p.sk_counter + rank * NWC + wave, 1);
+      ticket = __builtin_amdgcn_readfirstlane(ticket);
+      if (ticket != SPL - 1) continue;
+      for (int o = 0; o < SPL; ++o) {
+        if (o == sp) continue;
+        const int theirs = ((rank * SPL + o) * NWC + wave) * WAVE_BYTES + lane * 16;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const v4u v = __builtin_amdgcn_raw_buffer_load_b128(rP, theirs + ((i * TN + j) * 4 + q) * 1024, 0, SC1);
+              acc[i][j][4 * q] += (int)v[0]; acc[i][j][4 * q + 1] += (int)v[1];
+              acc[i][j][4 * q + 2] += (int)v[2]; acc[i][j][4 * q + 3] += (int)v[3];
+            }
+      }
+      if (lane == 0) atomicExch(p.sk_counter + rank * NWC + wave, 0);
     }
     stream_epilogue<TM, TN, OUTCLS>(p, e, acc, bz, m0 + wm * WTM, n0 + wn * WTN,
                                     lds + NSTAGE * STAGE + wave * (STRIP + COLS), lane);
@@ -1629,6 +1716,7 @@ struct Config {
   bool skinny = false;  // gemm_skinny_kernel: M <= 64, grid over 16-row slabs of B
   int stream_occ = 0;   // > 0: gemm_mfma_stream_kernel, this many workgroups per CU walk the tile list
   bool rows4 = false;   // gemm_rows4_kernel: M <= 16
+  int ws_waves = 0;     // > 0: gemm_mfma_ws_kernel with this many consumer waves (it can split K)
 };
 
 #define TI_FAST(BM, BN, BK, WM, WN, SWZ, NS)                                              \
@@ -1655,7 +1743,7 @@ struct Config {
         {gemm_mfma_ws_kernel<BM, BN, BK, WM, WN, SWZ, NS, OUT8, PW>,                        \
          gemm_mfma_ws_kernel<BM, BN, BK, WM, WN, SWZ, NS, OUT32, PW>,                       \
          gemm_mfma_ws_kernel<BM, BN, BK, WM, WN, SWZ, NS, OUT16, PW>},                      \
-        BM, BN, BK, (WM * WN + PW) * 64, true, false, 1                                   \
+        BM, BN, BK, (WM * WN + PW) * 64, true, false, 1, false, WM * WN                   \
   }
 
 enum ConfigId {
@@ -1673,6 +1761,7 @@ enum ConfigId {
   CFG_SKINNY_16_G2,  // M <= 16, a wave owns 2 slabs that share its A fragments
   CFG_ROWS4_16,      // M <= 16, K >= 1024: weights streamed as 1 KB row pieces
   CFG_WS_256x160,    // 2048 x 5120 outputs are exactly 256 of these tiles: one full round of the chip
+  CFG_WS_128x128,    // few activation rows and a long K: split K over enough of these to fill the chip
 };
 
 static const Config g_configs[] = {
@@ -1690,6 +1779,7 @@ static const Config g_configs[] = {
     {"skinny_m16_slab32", {gemm_skinny_kernel<OUT8, 1, 2>, gemm_skinny_kernel<OUT32, 1, 2>, gemm_skinny_kernel<OUT16, 1, 2>}, 16, 32, 64, 512, true, true},
     {"rows4_m16", {gemm_rows4_kernel<OUT8>, gemm_rows4_kernel<OUT32>, gemm_rows4_kernel<OUT16>}, 16, 4, 1024, (R4_NW + 1) * 64, true, false, 0, true},
     TI_WS(256, 160, 128, 4, 1, 1, 3, 4),
+    TI_WS(128, 128, 128, 2, 2, 1, 4, 4),
 };
 static const int g_num_configs = (int)(sizeof(g_configs) / sizeof(g_configs[0]));
 
@@ -1729,13 +1819,59 @@ static bool stream_eligible(const GemmParams& p) {
   return true;
 }
 
-// Tile choice: score = (measured relative efficiency of the tile class) x (fraction of the
-// 256 CUs kept busy over all rounds of workgroups) x (fraction of the tiles' area that is real
-// output) x (a small bonus for few rounds: a chip that is partly idle in its only round runs
-// that round faster than a full chip runs the first of two).  The class efficiencies were measured
-// with weights streamed from HBM.  Outputs the persistent kernels can store (row-major, aligned)
-// go to them; the rest to the one-tile kernels.
-static int pick_config(const GemmParams& p) {
+// k-tiles per split and the number of non-empty splits for `want` splits of a K of `kt` k-tiles
+static void sk_shape(int kt, int want, int& splits, int& kt_split) {
+  want = want < 1 ? 1 : (want > kt ? (kt > 0 ? kt : 1) : want);
+  kt_split = (kt + want - 1) / want;
+  splits = kt_split > 0 ? (kt + kt_split - 1) / kt_split : 1;
+}
+
+// Estimated run time (arbitrary unit) of the GEMM on configuration k with `want` K splits:
+//   rounds of work items over the chip's workgroup slots
+//   x the K bytes an item walks, plus a fixed part per item (pipeline fill, epilogue and store: about
+//     four k-tiles' worth) and, when K is split, the exchange of partial sums (the store of an
+//     item's sums plus, for the last item of a tile, one read per other split: measured about
+//     1 + 2.6 us per split for a 256 x 128 tile, i.e. four plus six k-tiles' worth per split)
+//   x the tile's outputs / the measured relative efficiency of the tile class (per slot)
+// with a small bonus for few rounds (a chip that is partly idle in its only round runs that round
+// faster than a full chip runs the first of two).  Padded parts of edge tiles cost like real ones.
+static double config_cost(const GemmParams& p, const Config& k, double eff, int want, int& splits) {
+  const int occ = k.stream_occ > 1 ? k.stream_occ : 1;
+  const int slots = 256 * occ;
+  const int64_t tm = (p.M + k.bm - 1) / k.bm, tn = (p.N + k.bn - 1) / k.bn;
+  const int kt = (p.K + k.bk - 1) / k.bk;
+  int kt_split = kt;
+  splits = 1;
+  if (want > 1 && k.ws_waves && p.batch == 1) sk_shape(kt, want, splits, kt_split);
+  const int64_t items = tm * tn * p.batch * splits;
+  const int64_t rounds = (items + slots - 1) / slots;
+  const double k_len = (double)kt_split * k.bk + 512.0 + (splits > 1 ? 512.0 + 768.0 * splits : 0.0);
+  return (double)rounds * k_len * (double)(k.bm * k.bn) * occ / eff / (1.0 + 0.1 / (double)rounds);
+}
+
+// Number of K splits for a wave-specialised configuration: as many as fill the chip's 256 workgroup
+// slots once, but no split shorter than 2048 bytes of K and no more than 8 (the last item of a tile
+// reads the other splits' sums one after the other).
+static int pick_splits(const GemmParams& p, const Config& k, double eff, double* cost_out) {
+  int want = 1;
+  if (k.ws_waves && p.batch == 1) {
+    const int64_t tiles = (int64_t)((p.M + k.bm - 1) / k.bm) * ((p.N + k.bn - 1) / k.bn);
+    const int64_t fill = tiles > 0 ? 256 / tiles : 1;
+    const int by_k = p.K / 2048;
+    want = (int)(fill < by_k ? fill : by_k);
+    want = want < 1 ? 1 : (want > 8 ? 8 : want);
+  }
+  int used = 1;
+  const double cost = config_cost(p, k, eff, want, used);
+  if (cost_out) *cost_out = cost;
+  return used;
+}
+
+// Tile choice: the configuration (and K split) with the lowest estimated run time.  The class
+// efficiencies were measured with weights streamed from HBM.  Outputs the persistent kernels can
+// store (row-major, aligned) go to them; the rest to the one-tile kernels.
+static int pick_config(const GemmParams& p, int* splits_out) {
+  *splits_out = 1;
   if (!fast_eligible(p)) return CFG_GATHER;
   if (p.M <= 16) {
     // one GEMM over a long K: stream the weights as whole row pieces; short K or batched (the
@@ -1743,31 +1879,34 @@ static int pick_config(const GemmParams& p) {
     if (p.batch <= 4 && p.K >= 1024) return CFG_ROWS4_16;
     return (p.N + 31) / 32 >= 160 ? CFG_SKINNY_16_G2 : CFG_SKINNY_16;
   }
-  if (p.M <= 64) return CFG_SKINNY_16 + (p.M > 16) + (p.M > 32);
   const bool stream = stream_eligible(p);
+  if (p.M <= 128 && stream && p.batch == 1 && p.K >= 1024) {
+    // a few rows against a long K: the GEMM is a read of the weight matrix.  128 x 128 tiles with K
+    // split over enough workgroups to have every CU pulling its own slab keep the most weight bytes
+    // in flight (measured, weights from HBM, N = 6848, K = 10240: M = 64 55 -> 29 us against the
+    // 16-row slabs, M = 128 52 -> 28 us against 64 x 64 tiles)
+    *splits_out = pick_splits(p, g_configs[CFG_WS_128x128], 1.0, nullptr);
+    return CFG_WS_128x128;
+  }
+  if (p.M <= 64) return CFG_SKINNY_16 + (p.M > 16) + (p.M > 32);
   // short K: the epilogue dominates and the larger tile halves the operand traffic per output
   const double big = p.K <= 512 ? 1.20 : 0.97;
-  struct Cand { int cfg; double base; };
+  struct Cand { int cfg; double eff; };
   const Cand cands[] = {
       {stream ? CFG_STREAM_256x256 : CFG_TILE_256x256, stream ? big : 1.00},
       {stream ? CFG_WS_256x128 : CFG_TILE_256x128, stream ? 1.00 : 0.90},
       {stream ? CFG_STREAM_128x128 : CFG_TILE_128x128, 0.78},
-      {CFG_TILE_64x64, 0.50},
+      {CFG_TILE_64x64, 0.25},
       {stream ? CFG_WS_256x160 : -1, 1.00},
+      {stream ? CFG_WS_128x128 : -1, 0.85},
   };
   int best = CFG_TILE_64x64;
-  double best_score = -1.0;
+  double best_cost = -1.0;
   for (const Cand& c : cands) {
     if (c.cfg < 0) continue;
-    const Config& k = g_configs[c.cfg];
-    const int slots = 256 * (k.stream_occ > 1 ? k.stream_occ : 1);
-    const int64_t tm = (p.M + k.bm - 1) / k.bm, tn = (p.N + k.bn - 1) / k.bn;
-    const int64_t tiles = tm * tn * p.batch;
-    const int64_t rounds = (tiles + slots - 1) / slots;
-    const double busy = (double)tiles / (double)(rounds * slots);
-    const double area = ((double)p.M * p.N) / ((double)(tm * k.bm) * (double)(tn * k.bn));
-    const double score = c.base * busy * area * (1.0 + 0.1 / (double)rounds);
-    if (score > best_score) best_score = score, best = c.cfg;
+    double cost;
+    const int splits = pick_splits(p, g_configs[c.cfg], c.eff, &cost);
+    if (best_cost < 0 || cost < best_cost) best_cost = cost, best = c.cfg, *splits_out = splits;
   }
   return best;
 }
@@ -1780,9 +1919,12 @@ static int pick_group_m(const GemmParams& p, const Config& k) {
   const int per_xcd = (int)((tiles + 7) / 8) < at_once ? (int)((tiles + 7) / 8) : at_once;
   int best = 1;
   int64_t best_cost = -1;
-  for (int g = 1; g <= p.tiles_m && g <= 64; g *= 2) {
+  // powers of two, and all of a short column of row tiles (3 or 6 row tiles in groups of 2 or 4
+  // would send the odd ones through the weight panels a second time)
+  for (int g = 1; g <= p.tiles_m && g <= 64; g = (g * 2 > p.tiles_m && g < p.tiles_m && p.tiles_m <= 64) ? p.tiles_m : g * 2) {
     const int cols = (per_xcd + g - 1) / g;
-    const int64_t cost = (int64_t)g * k.bm + (int64_t)cols * k.bn;
+    const int passes = (p.tiles_m + g - 1) / g;  // a short last group still walks all weight panels
+    const int64_t cost = ((int64_t)g * k.bm + (int64_t)cols * k.bn) * passes * g / p.tiles_m;
     if (best_cost < 0 || cost < best_cost) best_cost = cost, best = g;
   }
   return best;
@@ -1819,8 +1961,59 @@ static int validate(const GemmParams& p) {
 }
 
 static thread_local int g_last_config = -1;
+static thread_local int g_last_splits = 1;
 
+// ---- split-K workspace -----------------------------------------------------------------------------
+// One allocation per (device, stream): ticket counters (zeroed once; every launch leaves them at
+// zero) followed by the items' int32 partial sums.  Launches on one stream run one after the other,
+// so they can share it; launches on different streams may overlap and get their own.  It grows on
+// demand.
+constexpr size_t SK_COUNTER_INTS = 1 << 16;             // tiles x consumer waves of one launch
+constexpr size_t SK_MAX_PARTIAL_BYTES = (size_t)96 << 20;  // < 2 GiB: the kernel addresses it with 32-bit offsets
+struct SkWorkspace { int dev; hipStream_t stream; char* base; size_t partial_bytes; };
+static std::mutex g_sk_mutex;
+static std::vector<SkWorkspace> g_sk_ws;
+
+// 0 and the pointers, or a status.  With allocate == false (the stream is being captured into a
+// graph: no allocation possible) an existing workspace that is large enough is used, else TI_E_COMBO.
+static int sk_workspace(hipStream_t stream, size_t partial_bytes, bool allocate, int** partial, int** counter) {
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return fail((int)err, "hipGetDevice: %s", hipGetErrorString(err));
+  std::lock_guard<std::mutex> lock(g_sk_mutex);
+  SkWorkspace* w = nullptr;
+  for (auto& e : g_sk_ws)
+    if (e.dev == dev && e.stream == stream) w = &e;
+  if (!w || w->partial_bytes < partial_bytes) {
+    if (!allocate) return TI_E_COMBO;
+    // An outgrown workspace is not freed: a captured graph may hold its address.  Growing at least
+    // doubles it, so what stays behind is less than the final size.
+    if (w && partial_bytes < 2 * w->partial_bytes) partial_bytes = 2 * w->partial_bytes;
+    if (partial_bytes > SK_MAX_PARTIAL_BYTES) partial_bytes = SK_MAX_PARTIAL_BYTES;
+    char* base = nullptr;
+    const size_t bytes = SK_COUNTER_INTS * sizeof(int) + partial_bytes;
+    err = hipMalloc((void**)&base, bytes);
+    if (err == hipSuccess) err = hipMemset(base, 0, SK_COUNTER_INTS * sizeof(int));
+    if (err != hipSuccess) return fail((int)err, "split-K workspace of %zu bytes: %s", bytes, hipGetErrorString(err));
+    if (!w) {
+      g_sk_ws.push_back({dev, stream, nullptr, 0});
+      w = &g_sk_ws.back();
+    }
+    w->base = base;
+    w->partial_bytes = partial_bytes;
+  }
+  *counter = (int*)w->base;
+  *partial = (int*)(w->base + SK_COUNTER_INTS * sizeof(int));
+  return TI_OK;
+}
+
+
+// `config`: bits 0..7 the configuration (0xff or a negative value: choose), bits 8..15 the number of
+// K splits to use with a wave-specialised configuration (0: choose).
 static int run(GemmParams p, int config, hipStream_t stream) {
+  g_last_splits = 1;
+  int want_splits = config < 0 ? 0 : (config >> 8) & 0xff;
+  if (config >= 0) config = (config & 0xff) == 0xff ? -1 : (config & 0xff);
   int rc = validate(p);
   if (rc != TI_OK) return rc;
   if (p.batch == 0 || p.M == 0 || p.N == 0) return TI_OK;
@@ -1830,7 +2023,13 @@ static int run(GemmParams p, int config, hipStream_t stream) {
   // the fast kernels quantise to int8 with round-half-even only; the truncating test switch runs
   // on the gather kernel
   const bool trunc8 = p.round_mode == TI_ROUND_TRUNC && out_class(p.out_dtype) == OUT8;
-  if (config < 0) config = (trunc8 && p.M > 64) ? CFG_GATHER : pick_config(p);
+  int auto_splits = 1;
+  if (config < 0) {
+    // int8 truncation (a test-time switch) is implemented by the gather kernel and the M <= 64 kernels
+    if (trunc8 && p.M > 16) config = (p.M <= 64 && fast_eligible(p)) ? CFG_SKINNY_16 + 1 + (p.M > 32) : CFG_GATHER;
+    else config = pick_config(p, &auto_splits);
+  }
+  else if (config < g_num_configs && !want_splits && g_configs[config].ws_waves) auto_splits = pick_splits(p, g_configs[config], 1.0, nullptr);
   if (config >= g_num_configs) return fail(TI_E_COMBO, "config %d out of range", config);
   const Config& k = g_configs[config];
   if (!k.fn[out_class(p.out_dtype)]) return fail(TI_E_COMBO, "config %s has no kernel for output dtype %d", k.name, p.out_dtype);
@@ -1874,8 +2073,32 @@ static int run(GemmParams p, int config, hipStream_t stream) {
   if ((int64_t)p.tiles_m * p.tiles_n > 0x7fffffff) return fail(TI_E_SHAPE, "too many tiles");
   p.group_m = pick_group_m(p, k);
   g_last_config = config;
+  p.splits = 1;
+  p.kt_split = 0;
+  if (want_splits > 1 && !(k.ws_waves && p.batch == 1)) return fail(TI_E_COMBO, "config %s cannot split K (batch %d)", k.name, p.batch);
+  if (k.ws_waves && p.batch == 1) {
+    const int kt = (p.K + k.bk - 1) / k.bk;
+    const int64_t tiles = (int64_t)p.tiles_m * p.tiles_n;
+    int splits = want_splits ? want_splits : auto_splits;
+    sk_shape(kt, splits, splits, p.kt_split);
+    const size_t item_bytes = (size_t)k.bm * k.bn * sizeof(int);
+    if (splits > 1 && ((size_t)tiles * k.ws_waves > SK_COUNTER_INTS || (size_t)tiles * splits * item_bytes > SK_MAX_PARTIAL_BYTES)) {
+      if (want_splits) return fail(TI_E_SHAPE, "%d splits of %lld tiles exceed the split-K workspace", splits, (long long)tiles);
+      splits = 1;
+    }
+    if (splits > 1) {
+      hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+      (void)hipStreamIsCapturing(stream, &cap);
+      rc = sk_workspace(stream, (size_t)tiles * splits * item_bytes, cap == hipStreamCaptureStatusNone, &p.sk_partial, &p.sk_counter);
+      if (rc == TI_E_COMBO && !want_splits) splits = 1;  // capturing and nothing allocated yet: run unsplit
+      else if (rc == TI_E_COMBO) return fail(TI_E_COMBO, "no split-K workspace on this stream and none can be allocated during graph capture");
+      else if (rc != TI_OK) return rc;
+    }
+    p.splits = splits;
+  }
+  g_last_splits = p.splits;
   if (k.stream_occ) {
-    const int64_t items = (int64_t)p.tiles_m * p.tiles_n * p.batch;
+    const int64_t items = (int64_t)p.tiles_m * p.tiles_n * p.batch * p.splits;
     if (items > 0x7fffffff) return fail(TI_E_SHAPE, "too many tiles");
     int64_t g = items < 256 * k.stream_occ ? items : 256 * k.stream_occ;
     if (g >= 8) g &= ~(int64_t)7;  // a multiple of 8 keeps workgroup b on XCD b % 8
@@ -1917,13 +2140,14 @@ static int run_with_residual(GemmParams p, const float* R, int64_t ldr, hipStrea
   rc = check_device();
   if (rc != TI_OK) return rc;
   if (!p.bias) p.bias_kind = TI_BIAS_NONE;
-  const int cfg = pick_config(p);
+  int splits = 1;
+  const int cfg = pick_config(p, &splits);
   if (g_configs[cfg].rows4) {  // the decode kernel adds the residual in its store phase
     p.resid = R;
     p.resid_rs = ldr;
     return run(p, cfg, stream);
   }
-  rc = run(p, cfg, stream);
+  rc = run(p, cfg | (splits << 8), stream);
   if (rc != TI_OK) return rc;
   const int vec = (p.N % 4 == 0) && (p.sCm % 4 == 0) && (ldr % 4 == 0) && (((uintptr_t)p.C | (uintptr_t)R) & 15) == 0;
   const int64_t items = (int64_t)p.M * (vec ? p.N / 4 : p.N);
@@ -1953,6 +2177,7 @@ int ti_bmm_i8_config(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk, con
   p.bias_bs = 0; p.scale_bs = 0;
   p.resid = nullptr; p.resid_rs = 0;
   p.kv_k = p.kv_vt = nullptr; p.kv_k_hs = p.kv_vt_rs = 0; p.kv_D = 1;
+  p.splits = 1; p.kt_split = 0; p.sk_partial = p.sk_counter = nullptr;
   return ti::run(p, config, (hipStream_t)stream);
 }
 
@@ -1975,6 +2200,7 @@ int ti_bmm_i8_grouped(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk, co
   p.bias_bs = bias_batch_stride; p.scale_bs = scale_batch_stride;
   p.resid = nullptr; p.resid_rs = 0;
   p.kv_k = p.kv_vt = nullptr; p.kv_k_hs = p.kv_vt_rs = 0; p.kv_D = 1;
+  p.splits = 1; p.kt_split = 0; p.sk_partial = p.sk_counter = nullptr;
   return ti::run(p, config, (hipStream_t)stream);
 }
 
@@ -1999,12 +2225,14 @@ int ti_qkv_decode_i8(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw,
   p.bias_bs = N; p.scale_bs = 1;
   p.resid = nullptr; p.resid_rs = 0;
   p.kv_k = k_dst; p.kv_vt = vt_dst; p.kv_k_hs = k_head_stride; p.kv_vt_rs = vt_row_stride; p.kv_D = D;
+  p.splits = 1; p.kt_split = 0; p.sk_partial = p.sk_counter = nullptr;
   int rc = validate(p);
   if (rc != TI_OK) return rc;
   if (M == 0 || N == 0) return TI_OK;
   rc = check_device();
   if (rc != TI_OK) return rc;
-  const int cfg = pick_config(p);
+  int splits = 1;
+  const int cfg = pick_config(p, &splits);
   if (!g_configs[cfg].rows4) return fail(TI_E_COMBO, "operands not eligible for the decode kernel (16-byte aligned, K-contiguous)");
   return run(p, cfg, (hipStream_t)stream);
 }
@@ -2033,6 +2261,7 @@ int ti_linear_i8_residual_f32(const int8_t* A, int64_t lda, const int8_t* W, int
   p.bias_bs = 0; p.scale_bs = 0;
   p.resid = nullptr; p.resid_rs = 0;
   p.kv_k = p.kv_vt = nullptr; p.kv_k_hs = p.kv_vt_rs = 0; p.kv_D = 1;
+  p.splits = 1; p.kt_split = 0; p.sk_partial = p.sk_counter = nullptr;
   return ti::run_with_residual(p, residual, ldr, (hipStream_t)stream);
 }
 
@@ -2040,6 +2269,8 @@ int ti_linear_i8_residual_f32(const int8_t* A, int64_t lda, const int8_t* W, int
 int ti_gemm_num_configs(void) { return ti::g_num_configs; }
 
 int ti_gemm_last_config(void) { return ti::g_last_config; }
+
+int ti_gemm_last_splits(void) { return ti::g_last_splits; }
 
 const char* ti_gemm_config_name(int config) {
   return (config >= 0 && config < ti::g_num_configs) ? ti::g_configs[config].name : "";
