@@ -152,6 +152,29 @@ int ti_bmm_i8_grouped(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk,
                       const float* alpha, const float* beta, int64_t scale_batch_stride,
                       int epilogue, int out_dtype, int round_mode,
                       int config, void* stream);
+/*
+ * ti_bmm_i8_config for callers that cannot allocate device memory (a stream under HIP graph capture
+ * before any workspace exists, a serving loop or harness that forbids hipMalloc).  It has no
+ * counterpart in the reference.  Same arguments, same arithmetic, same kernels and the same choice
+ * of configuration and K split as ti_bmm_i8_config; the difference is where a split-K launch keeps
+ * its ticket counters and int32 partial sums: in a fixed array in the library's device image
+ * (16384 counters + 32 MiB of partial sums, held by every GPU the library runs on until the process
+ * ends) instead of the per-stream workspace ti_bmm_i8 allocates.  The call allocates and frees
+ * nothing, on the host side of the device or through any library.  A launch whose partial sums
+ * would not fit (tiles x splits x tile bytes > 32 MiB, or tiles x 4 > 16384) returns TI_E_SHAPE and
+ * launches nothing; launches that do not split K use no scratch and always fit.  All calls on one
+ * GPU share that GPU's array: two calls that may run at the same time on one GPU (different
+ * streams, different host threads) race on it and must be serialised by the caller.  Kernels leave
+ * the counters at zero; the partial sums are overwritten before they are read.
+ */
+int ti_bmm_i8_static_scratch(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk,
+                             const int8_t* B, int64_t sBb, int64_t sBn, int64_t sBk,
+                             void* C, int64_t sCb, int64_t sCm, int64_t sCn,
+                             int batch, int M, int N, int K,
+                             const void* bias, int bias_kind,
+                             const float* alpha, const float* beta,
+                             int epilogue, int out_dtype, int round_mode,
+                             int config, void* stream);
 int ti_gemm_num_configs(void);
 const char* ti_gemm_config_name(int config);
 /* Index of the configuration the calling thread's most recent ti_bmm_i8* launch used (-1 if

@@ -2008,9 +2008,50 @@ static int sk_workspace(hipStream_t stream, size_t partial_bytes, bool allocate,
 }
 
 
+// ---- split-K scratch that needs no allocation ---------------------------------------------------------
+// For callers that cannot allocate (a stream under graph capture, a serving loop that forbids it):
+// the same layout as the allocated workspace, ticket counters followed by partial sums, in a
+// file-scope device array of fixed size.  Every GPU the library runs on holds its own copy for the
+// life of the process.  Host code never uses the array's name as an address: its device address
+// is looked up once per device, with that device current, and that pointer is what kernels get.
+constexpr size_t SK_STATIC_COUNTER_INTS = 1 << 14;            // tiles x consumer waves of one launch
+constexpr size_t SK_STATIC_PARTIAL_BYTES = (size_t)32 << 20;  // 256 work items of a 256 x 128 tile
+constexpr size_t SK_STATIC_INTS = SK_STATIC_COUNTER_INTS + SK_STATIC_PARTIAL_BYTES / sizeof(int);
+static __device__ __align__(256) int scratch[SK_STATIC_INTS];
+static int* g_scratch_ptr[64];
+
+__global__ __launch_bounds__(256) void sk_clear_counters_kernel(int* counters, int n) {
+  for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) counters[i] = 0;
+}
+
+// Device address of the calling thread's current device's copy of `scratch`.  First call on a
+// device: looks the address up and zero-fills the ticket counters with a small kernel on `stream`
+// (launches leave them at zero afterwards); no allocation, no memset node.
+static int sk_static_scratch(hipStream_t stream, int** partial, int** counter) {
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return fail((int)err, "hipGetDevice: %s", hipGetErrorString(err));
+  if (dev < 0 || dev >= 64) return fail(TI_E_DEVICE, "device index %d beyond the %d the static scratch table covers", dev, 64);
+  std::lock_guard<std::mutex> lock(g_sk_mutex);
+  if (!g_scratch_ptr[dev]) {
+    int* ptr = nullptr;
+    err = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || !ptr) return fail(err != hipSuccess ? (int)err : TI_E_NULL, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(err));
+    sk_clear_counters_kernel<<<dim3(16), dim3(256), 0, stream>>>(ptr, (int)SK_STATIC_COUNTER_INTS);
+    const int rc = launch_status("sk_clear_counters_kernel");
+    if (rc != TI_OK) return rc;
+    g_scratch_ptr[dev] = ptr;
+  }
+  *counter = g_scratch_ptr[dev];
+  *partial = g_scratch_ptr[dev] + SK_STATIC_COUNTER_INTS;
+  return TI_OK;
+}
+
 // `config`: bits 0..7 the configuration (0xff or a negative value: choose), bits 8..15 the number of
 // K splits to use with a wave-specialised configuration (0: choose).
-static int run(GemmParams p, int config, hipStream_t stream) {
+// static_scratch: split-K launches use the fixed device array instead of the allocated workspace, and a
+// launch whose partial sums do not fit it is refused (nothing is allocated or freed on this path).
+static int run(GemmParams p, int config, hipStream_t stream, bool static_scratch = false) {
   g_last_splits = 1;
   int want_splits = config < 0 ? 0 : (config >> 8) & 0xff;
   if (config >= 0) config = (config & 0xff) == 0xff ? -1 : (config & 0xff);
@@ -2082,11 +2123,18 @@ static int run(GemmParams p, int config, hipStream_t stream) {
     int splits = want_splits ? want_splits : auto_splits;
     sk_shape(kt, splits, splits, p.kt_split);
     const size_t item_bytes = (size_t)k.bm * k.bn * sizeof(int);
-    if (splits > 1 && ((size_t)tiles * k.ws_waves > SK_COUNTER_INTS || (size_t)tiles * splits * item_bytes > SK_MAX_PARTIAL_BYTES)) {
+    if (splits > 1 && static_scratch) {
+      if ((size_t)tiles * k.ws_waves > SK_STATIC_COUNTER_INTS || (size_t)tiles * splits * item_bytes > SK_STATIC_PARTIAL_BYTES)
+        return fail(TI_E_SHAPE, "%d K splits of %lld tiles need %zu bytes of partial sums: more than the %zu bytes of static scratch "
+                    "(use ti_bmm_i8, which allocates its workspace)", splits, (long long)tiles, (size_t)tiles * splits * item_bytes,
+                    SK_STATIC_PARTIAL_BYTES);
+      rc = sk_static_scratch(stream, &p.sk_partial, &p.sk_counter);
+      if (rc != TI_OK) return rc;
+    } else if (splits > 1 && ((size_t)tiles * k.ws_waves > SK_COUNTER_INTS || (size_t)tiles * splits * item_bytes > SK_MAX_PARTIAL_BYTES)) {
       if (want_splits) return fail(TI_E_SHAPE, "%d splits of %lld tiles exceed the split-K workspace", splits, (long long)tiles);
       splits = 1;
     }
-    if (splits > 1) {
+    if (splits > 1 && !static_scratch) {
       hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
       (void)hipStreamIsCapturing(stream, &cap);
       rc = sk_workspace(stream, (size_t)tiles * splits * item_bytes, cap == hipStreamCaptureStatusNone, &p.sk_partial, &p.sk_counter);
@@ -2243,6 +2291,27 @@ int ti_bmm_i8(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk, const int8
               int round_mode, void* stream) {
   return ti_bmm_i8_config(A, sAb, sAm, sAk, B, sBb, sBn, sBk, C, sCb, sCm, sCn, batch, M, N, K, bias, bias_kind,
                           alpha, beta, epilogue, out_dtype, round_mode, -1, stream);
+}
+
+int ti_bmm_i8_static_scratch(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk, const int8_t* B, int64_t sBb, int64_t sBn,
+                             int64_t sBk, void* C, int64_t sCb, int64_t sCm, int64_t sCn, int batch, int M, int N, int K,
+                             const void* bias, int bias_kind, const float* alpha, const float* beta, int epilogue,
+                             int out_dtype, int round_mode, int config, void* stream) {
+  ti::GemmParams p;
+  p.A = A; p.B = B; p.C = C;
+  p.sAb = sAb; p.sAm = sAm; p.sAk = sAk;
+  p.sBb = sBb; p.sBn = sBn; p.sBk = sBk;
+  p.sCb = sCb; p.sCm = sCm; p.sCn = sCn;
+  p.batch = batch; p.M = M; p.N = N; p.K = K;
+  p.bias = bias; p.bias_kind = bias_kind;
+  p.alpha = alpha; p.beta = beta;
+  p.epilogue = epilogue; p.out_dtype = out_dtype; p.round_mode = round_mode;
+  p.tiles_m = p.tiles_n = 0; p.group_m = 1; p.ksplit = 1;
+  p.bias_bs = 0; p.scale_bs = 0;
+  p.resid = nullptr; p.resid_rs = 0;
+  p.kv_k = p.kv_vt = nullptr; p.kv_k_hs = p.kv_vt_rs = 0; p.kv_D = 1;
+  p.splits = 1; p.kt_split = 0; p.sk_partial = p.sk_counter = nullptr;
+  return ti::run(p, config, (hipStream_t)stream, true);
 }
 
 int ti_linear_i8_residual_f32(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw, const float* bias,
