@@ -416,7 +416,8 @@ def test_split_k_every_ws_config_bit_exact(M, N, K):
             for _ in range(2):
                 assert np.array_equal(cpu(linear.linear_a8_w8_b32_o32(ga, gw, gb32, _config=forced)), want32), (name, splits)
                 used = L.lib().ti_gemm_last_splits()
-                assert 1 < used <= min(splits, (K + 127) // 128), (name, splits, used)
+                bk = int(name.split("_")[1].split("x")[2])
+                assert 1 < used <= min(splits, (K + bk - 1) // bk), (name, splits, used)
                 assert np.array_equal(cpu(linear.linear_a8_w8_b8_o8(ga, gw, gb8, alpha, beta, _config=forced)), want8), (name, splits)
                 assert np.array_equal(cpu(linear.linear_a8_w8_bfp32_ofp32(ga, gw, gbf, alpha, 1.0, _config=forced)), wantf), (name, splits)
             ran += 1

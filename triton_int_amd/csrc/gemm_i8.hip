@@ -197,6 +197,31 @@ __device__ __forceinline__ EpiCtx make_epi(const GemmParams& p, int bz) {
   return e;
 }
 
+// ---- int8 quantisation of 16 clamped fp32 values into 4 dwords --------------------------------
+// v + 1.5 * 2^23 rounds v to the nearest integer (ties to even) and leaves the two's-complement
+// int8 in the low byte of the sum's bit pattern (|v| <= 128 after the clamp).  The adds write that
+// byte straight into byte t of dword g (sub-dword destination select, the other bytes preserved),
+// so there is no separate packing step: 4 instead of 4.75 vector instructions per output.  The
+// four dwords are interleaved because a partial write must not be read by the very next
+// instruction; the trailing s_nop covers whatever instruction follows the block.
+__device__ __forceinline__ void pack16_q8(const float (&f)[4][4], unsigned (&X)[4]) {
+  const float magic = 12582912.0f;
+#define TI_SDWA_ADD(G, T, B) "v_add_f32_sdwa %" #G ", %4, %" #T " dst_sel:" B " dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD\n\t"
+  asm("v_add_f32_e32 %0, %4, %5\n\t"
+      "v_add_f32_e32 %1, %4, %9\n\t"
+      "v_add_f32_e32 %2, %4, %13\n\t"
+      "v_add_f32_e32 %3, %4, %17\n\t"
+      TI_SDWA_ADD(0, 6, "BYTE_1") TI_SDWA_ADD(1, 10, "BYTE_1") TI_SDWA_ADD(2, 14, "BYTE_1") TI_SDWA_ADD(3, 18, "BYTE_1")
+      TI_SDWA_ADD(0, 7, "BYTE_2") TI_SDWA_ADD(1, 11, "BYTE_2") TI_SDWA_ADD(2, 15, "BYTE_2") TI_SDWA_ADD(3, 19, "BYTE_2")
+      TI_SDWA_ADD(0, 8, "BYTE_3") TI_SDWA_ADD(1, 12, "BYTE_3") TI_SDWA_ADD(2, 16, "BYTE_3") TI_SDWA_ADD(3, 20, "BYTE_3")
+      "s_nop 0"
+      : "=&v"(X[0]), "=&v"(X[1]), "=&v"(X[2]), "=&v"(X[3])
+      : "v"(magic), "v"(f[0][0]), "v"(f[0][1]), "v"(f[0][2]), "v"(f[0][3]), "v"(f[1][0]), "v"(f[1][1]), "v"(f[1][2]),
+        "v"(f[1][3]), "v"(f[2][0]), "v"(f[2][1]), "v"(f[2][2]), "v"(f[2][3]), "v"(f[3][0]), "v"(f[3][1]), "v"(f[3][2]),
+        "v"(f[3][3]));
+#undef TI_SDWA_ADD
+}
+
 // ---- fast family -----------------------------------------------------------------------------
 //
 // LDS stage = A tile (BM x BK bytes) + B tile (BN x BK bytes), each viewed as 16-byte chunks;
@@ -468,12 +493,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
     auto body = [&](auto gelu_tag, auto bias_tag) {
       constexpr bool GELU = decltype(gelu_tag)::value;
       constexpr bool BIAS = decltype(bias_tag)::value;
-      auto one = [&](int a, float col) -> unsigned {
+      auto one = [&](int a, float col) -> float {
         float v = (float)a * e.alpha;
         if constexpr (BIAS) v = col + v;
         if constexpr (GELU) v = gelu_tanh_scaled(v, e.beta);
-        v = __builtin_amdgcn_fmed3f(v, q_floor, 127.0f);
-        return __float_as_uint(v + 12582912.0f);
+        return __builtin_amdgcn_fmed3f(v, q_floor, 127.0f);
       };
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
@@ -492,13 +516,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
           unsigned X[4];
+          float f[4][4];
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const unsigned b0 = one(acc[i][j][4 * g + 0], col[g][0]), b1 = one(acc[i][j][4 * g + 1], col[g][1]);
-            const unsigned b2 = one(acc[i][j][4 * g + 2], col[g][2]), b3 = one(acc[i][j][4 * g + 3], col[g][3]);
-            // low bytes of b0..b3 -> one dword
-            X[g] = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u) | __builtin_amdgcn_perm(b3, b2, 0x04000c0cu);
-          }
+          for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) f[g][t] = one(acc[i][j][4 * g + t], col[g][t]);
+          pack16_q8(f, X);
           const auto s02 = __builtin_amdgcn_permlane32_swap(X[0], X[2], false, false);
           const auto s13 = __builtin_amdgcn_permlane32_swap(X[1], X[3], false, false);
           v4u v;
@@ -627,26 +650,26 @@ __device__ __forceinline__ void stream_epilogue(const GemmParams& p, const EpiCt
         for (int c = lane; c < WTN; c += 64)
           cols[c] = column_term_t<GELU ? TI_BIAS_F32 : TI_BIAS_I8>(e, min(nw + c, p.N - 1), GELU);
       }
-      auto one = [&](int a, float col) -> unsigned {
+      auto one = [&](int a, float col) -> float {
         float v = (float)a * e.alpha;
         if constexpr (BIAS) v = col + v;
         if constexpr (GELU) v = gelu_tanh_scaled(v, e.beta);
-        v = __builtin_amdgcn_fmed3f(v, q_floor, 127.0f);
-        return __float_as_uint(v + 12582912.0f);
+        return __builtin_amdgcn_fmed3f(v, q_floor, 127.0f);
       };
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
           unsigned X[4];
+          float f[4][4];
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             v4f col = {0.f, 0.f, 0.f, 0.f};
             if constexpr (BIAS) col = *(const v4f*)(cols + j * 32 + 8 * g + 4 * lhi);
-            const unsigned b0 = one(acc[i][j][4 * g + 0], col[0]), b1 = one(acc[i][j][4 * g + 1], col[1]);
-            const unsigned b2 = one(acc[i][j][4 * g + 2], col[2]), b3 = one(acc[i][j][4 * g + 3], col[3]);
-            X[g] = __builtin_amdgcn_perm(b1, b0, 0x0c0c0400u) | __builtin_amdgcn_perm(b3, b2, 0x04000c0cu);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) f[g][t] = one(acc[i][j][4 * g + t], col[t]);
           }
+          pack16_q8(f, X);
           const auto s02 = __builtin_amdgcn_permlane32_swap(X[0], X[2], false, false);
           const auto s13 = __builtin_amdgcn_permlane32_swap(X[1], X[3], false, false);
           v4u v;
@@ -873,19 +896,23 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
     if (r < TM) fa[buf][r] = *(const v4i*)(stage + a_lane + r * 32 * BK + coff);
     else fb[buf][r - TM] = *(const v4i*)(stage + b_lane + (r - TM) * 32 * BK + coff);
   };
-  auto mfma = [&](int buf, int u) {
+  // first: the tile's first k-step starts from a zero C operand (an inline constant of the
+  // instruction) instead of accumulators cleared with one move each
+  auto mfma = [&](int buf, int u, auto first_tag) {
     const int i = u / TN, j = u % TN;
+    const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    const v16i c = decltype(first_tag)::value ? zero : acc[i][j];
     if constexpr (OUTCLS == OUT8)  // rows of the MFMA result = n (4 consecutive n per lane)
-      acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
+      acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[buf][j], fa[buf][i], c, 0, 0, 0);
     else  // rows of the MFMA result = m, lanes run along n
-      acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
+      acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[buf][i], fb[buf][j], c, 0, 0, 0);
   };
   constexpr int NM = TM * TN, NR = TM + TN;
-  auto kstep = [&](int buf, const char* rd_stage, int rd_ks, bool do_read, int d0, int nd) {
+  auto kstep = [&](int buf, const char* rd_stage, int rd_ks, bool do_read, int d0, int nd, auto first_tag) {
     int d = 0;
 #pragma unroll
     for (int u = 0; u < NM; ++u) {
-      mfma(buf, u);
+      mfma(buf, u, first_tag);
       if (do_read) {
 #pragma unroll
         for (int r = 0; r < NR; ++r)
@@ -921,12 +948,14 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
     int bz, m0, n0;
     locate(it, bz, m0, n0);
     const EpiCtx e = make_epi(p, bz);  // scalar loads, long done when the epilogue needs them
+    if (KT == 0) {  // K == 0: no MFMA defines the sums
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+          for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+    }
     // k-tile 0 of this item has landed: the barrier of the previous k-tile (or the one above) saw to it
 #pragma unroll
     for (int r = 0; r < NR; ++r) load_frag(lds + st * STAGE, 0, 0, r);
@@ -938,14 +967,15 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
       for (int ks = 0; ks < KS - 1; ++ks) {
         const int d0 = ks * PER_KS;
         const int nd = (d0 + PER_KS <= LOADS_A) ? PER_KS : (LOADS_A - d0 > 0 ? LOADS_A - d0 : 0);
-        kstep(ks & 1, cur, ks + 1, true, d0, nd);
+        if (ks == 0 && kt == 0) kstep(0, cur, 1, true, d0, nd, std::true_type{});  // starts the tile's sums
+        else kstep(ks & 1, cur, ks + 1, true, d0, nd, std::false_type{});
       }
       // all LDS reads of this k-tile are issued; the next k-tile must have landed before the
       // barrier.  The stores of the previous item's epilogue are younger than that k-tile while
       // it is one of those that were fetched before the epilogue.
       if (it > 0 && kt < DEPTH - 1) wait_loads_and_barrier<N_AFTER_STORES>();
       else wait_loads_and_barrier<N_STEADY>();
-      kstep((KS - 1) & 1, lds + st * STAGE, 0, kt + 1 < KT, LOADS_A, LOADS_B);
+      kstep((KS - 1) & 1, lds + st * STAGE, 0, kt + 1 < KT, LOADS_A, LOADS_B, std::false_type{});
       dma_advance();
     }
 
@@ -1140,24 +1170,29 @@ __global__ __launch_bounds__((WAVES_M * WAVES_N + PW) * 64) void gemm_mfma_ws_ke
     if (r < TM) fa[buf][r] = *(const v4i*)(stage + a_lane + r * 32 * BK + coff);
     else fb[buf][r - TM] = *(const v4i*)(stage + b_lane + (r - TM) * 32 * BK + coff);
   };
-  auto mfma = [&](int buf, int u) {
+  // first: the tile's first k-step starts from a zero C operand (an inline constant of the
+  // instruction) instead of accumulators cleared with one move each: 16 * TM * TN vector
+  // instructions per tile less, which is a seventh of the vector work of a K = 128 tile
+  auto mfma = [&](int buf, int u, auto first_tag) {
     const int i = u / TN, j = u % TN;
+    const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    const v16i c = decltype(first_tag)::value ? zero : acc[i][j];
     if constexpr (OUTCLS == OUT8)  // rows of the MFMA result = n (4 consecutive n per lane)
-      acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[buf][j], fa[buf][i], acc[i][j], 0, 0, 0);
+      acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[buf][j], fa[buf][i], c, 0, 0, 0);
     else  // rows of the MFMA result = m, lanes run along n
-      acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
+      acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[buf][i], fb[buf][j], c, 0, 0, 0);
   };
   constexpr int NM = TM * TN, NR = TM + TN;
   // One k-step, pinned order: MFMA u, then RPM fragment reads of the following k-step.  The reads go
   // out in the order in which the next k-step's MFMAs (i major, j minor) first touch a fragment:
   // A0, B0 .. B(TN-1), A1 .. A(TM-1), so that every fragment has most of a k-step of MFMAs between
   // its read and its first use (an LDS read takes longer than three MFMAs to come back).
-  auto kstep = [&](int buf, const char* rd_stage, int rd_ks, auto rpm_tag) {
+  auto kstep = [&](int buf, const char* rd_stage, int rd_ks, auto rpm_tag, auto first_tag) {
     constexpr int RPM_ = decltype(rpm_tag)::value;
     constexpr int RPM = RPM_ * NM >= NR ? RPM_ : (NR + NM - 1) / NM;
 #pragma unroll
     for (int u = 0; u < NM; ++u) {
-      mfma(buf, u);
+      mfma(buf, u, first_tag);
 #pragma unroll
       for (int s = u * RPM; s < (u + 1) * RPM; ++s)
         if (s < NR) {
@@ -1175,27 +1210,36 @@ __global__ __launch_bounds__((WAVES_M * WAVES_N + PW) * 64) void gemm_mfma_ws_ke
     int bz, m0, n0, rank, sp, kt0, kts;
     locate(it, bz, m0, n0, rank, sp, kt0, kts);
     const EpiCtx e = make_epi(p, bz);  // scalar loads, long done when the epilogue needs them
+    if (kts == 0) {  // K == 0: no MFMA defines the sums
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+          for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+    }
 #pragma unroll
     for (int r = 0; r < NR; ++r) load_frag(lds + st * STAGE, 0, 0, r);
     for (int kt = 0; kt < kts; ++kt) {
       const char* cur = lds + st * STAGE;
       st = (st + 1 == NSTAGE) ? 0 : st + 1;
+      // k-step 0 of the tile's first k-tile starts the sums; it is the k-step before the barrier when a
+      // k-tile has only two
+      if (KS > 2) {
+        if (kt == 0) kstep(0, cur, 1, Rpm1{}, std::true_type{});
+        else kstep(0, cur, 1, Rpm1{}, std::false_type{});
+      }
 #pragma unroll
-      for (int ks = 0; ks < KS - 2; ++ks) kstep(ks & 1, cur, ks + 1, Rpm1{});
+      for (int ks = 1; ks < KS - 2; ++ks) kstep(ks & 1, cur, ks + 1, Rpm1{}, std::false_type{});
       // the k-step before the barrier issues its reads early (two per MFMA), so that they have come
       // back when the barrier is reached
-      kstep((KS - 2) & 1, cur, KS - 1, RpmLast{});
+      if (KS == 2 && kt == 0) kstep(0, cur, 1, RpmLast{}, std::true_type{});
+      else kstep((KS - 2) & 1, cur, KS - 1, RpmLast{}, std::false_type{});
       // every LDS read of this k-tile is issued: wait for them, then hand the stage back
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
       // last k-step; the fragments it fetches are the first of the next k-tile (of the next item
       // after the last k-tile: landed as well, and simply fetched again at the item's start)
-      kstep((KS - 1) & 1, lds + st * STAGE, 0, Rpm1{});
+      kstep((KS - 1) & 1, lds + st * STAGE, 0, Rpm1{}, std::false_type{});
     }
     if (SPL > 1) {
       // Split K.  Each consumer wave settles its own quarter of the tile with the same wave of the
