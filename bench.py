@@ -397,6 +397,9 @@ def main():
     ap.add_argument("--attention-only", action="store_true",
                     help="run 3 full and 3 causal launches of the fused attention kernel (40 heads x 2048 x 2048 "
                          "x 128) and exit: the program profiled for the attention counter summary")
+    ap.add_argument("--bmm-qk-only", action="store_true",
+                    help="run 4 launches of the Q.K^T BMM to int8 (160 x 2048 x 2048 x 128) and exit: the program "
+                         "profiled for the Q.K^T counter summary")
     ap.add_argument("--calib-copy-mb", type=int, default=0,
                     help="before the timed region, run 4 device-to-device copies of this many MiB: a kernel of "
                          "known traffic to scale rocprofv3's FETCH_SIZE / WRITE_SIZE readings with")
@@ -423,6 +426,15 @@ def main():
         al, be = torch.tensor(0.002, device=dev), torch.tensor(0.01, device=dev)
         for i in range(24):
             linear.linear_a8_w8_b8_o8(x, ws[i % 6], b8, al, be)
+        torch.cuda.synchronize()
+        return
+    if args.bmm_qk_only:
+        from triton_int_amd.kernels import bmm
+
+        q, k = (torch.randint(-127, 128, (160, 2048, 128), dtype=torch.int8, device=dev) for _ in range(2))
+        sc = torch.empty((160, 2048, 2048), dtype=torch.int8, device=dev)
+        for _ in range(4):
+            bmm.bmm_s8t_s8n_s8t(q, k, 1e-3, out=sc)
         torch.cuda.synchronize()
         return
     if args.attention_only:
