@@ -234,8 +234,14 @@ int ti_gelu_q(const float* x, const float* scale, int8_t* y, int64_t n,
  * The link between the two attention BMMs of a W8A8 decoder layer: int8 scores from
  * bmm_s8t_s8n_s8t (kernels/bmm.py:576-612) in, int8 probabilities for the P.V BMM out.  The
  * reference tree has no kernel for it (its modules stop at the BMMs); the arithmetic is the
- * fp32 softmax followed by `mul(127).round()` that SmoothQuant-style callers of these modules do.
- * scale is a host float (score scale).  causal_q_len > 0: rows come in groups of that many query
+ * fp32 softmax followed by `mul(127).round()` that SmoothQuant-style callers of these modules do,
+ * fixed as follows so that every kernel that forms these probabilities (this one and
+ * ti_attention_i8) gives the same bits whatever order it visits a row in:
+ *     mx = largest visible score of the row;  s2 = scale * log2(e)  (fp32)
+ *     e_j = exp2(fma(float(x_j), s2, -(float(mx) * s2)))
+ *     S   = sum_j round_half_even(e_j * 2^23)              an integer: exact in any order
+ *     y_j = round_half_even(e_j * (127 * 2^23 / float(S)))     float(S) correctly rounded, IEEE division
+ * scale is a host float (score scale), >= 0.  causal_q_len > 0: rows come in groups of that many query
  * positions, position i attends to columns 0 .. i + (cols - causal_q_len); 0 = no mask.
  * cols <= 8192.  Row strides in elements, unit column stride.
  */
@@ -300,14 +306,12 @@ int ti_kv_append_i8(const int8_t* k_src, int64_t k_src_row_stride, const int8_t*
  *     out    = q8(pv_alpha * (probs . v))                  (bmm_s8t_s8n_s8t again, b = V^T)
  * q [batch, S, D], k [batch, T, D], vt [batch, D, T] (V^T, as the P.V BMM takes it), out
  * [batch, S, D]; int8, unit stride along the last dimension, batch and row strides in elements
- * (all multiples of 16, like the pointers); D = 128; T a multiple of 16; 0 < score_scale <= 0.32.
- * The scalars are host floats.  The int8 scores are bit-identical to the BMM's; a probability can
- * differ from ti_softmax_q's by one step where 127 * e / sum lies within fp32 rounding of a half
- * (the row's exponentials are summed in a different order).  All columns of a row that share an
- * int8 score flip together, so such a row (about 1 in 10^5 at 2048 keys) can differ from the
- * three-launch result in several output values by a few steps; every other row is identical.
+ * (all multiples of 16, like the pointers); D = 128; T a multiple of 16; score_scale > 0.
+ * The scalars are host floats.  The int8 scores are the BMM's and the probabilities ti_softmax_q's
+ * bit for bit (a row's exponentials are summed as integers, so the order in which the keys are
+ * visited does not matter): the output equals the three-launch chain's exactly.
  * With S <= 16 and T <= 4096 (decode) a one-pass kernel runs instead, one to four workgroups per
- * batch entry; it takes the exponent against the row maximum like ti_softmax_q.
+ * batch entry.
  * The reference has no fused form (its modules stop at the BMMs, nn/bmm.py:10-74); the
  * three-launch chain remains available and is what this is tested against.
  */

@@ -265,14 +265,23 @@ int ti_oracle_gelu_q(const float* x, const float* scale, int8_t* y, int64_t n, i
   return 0;
 }
 
-/* int8 scores -> int8 probabilities: fp32 softmax of x*scale over the row (max-subtracted, libm expf,
- * division per element), then round_half_even(p * 127) — `softmax(...).mul(127).round()` as
+/* int8 scores -> int8 probabilities round_half_even(127 * softmax(x * scale)) over the row, as
  * SmoothQuant-style callers of the BMM modules do between bmm_s8t_s8n_s8t (kernels/bmm.py:576-612)
- * and the P.V BMM; the reference tree itself has no such function, so there is nothing of the
- * reference's to follow line by line.  Pins: torch.softmax on x*scale, mul(127), round
- * (tests/test_oracle_rowops.py).  causal_q_len as in the HIP entry point. */
+ * and the P.V BMM (`softmax(...).mul(127).round()`); the reference tree itself has no such function,
+ * so there is nothing of the reference's to follow line by line.  The fp32 steps are fixed so that
+ * the row sum does not depend on the order of summation (the HIP kernels visit a row in different
+ * orders and must agree with each other bit for bit):
+ *     mx = largest visible score;  s2 = scale * log2(e)
+ *     e_j = exp2f(fmaf((float)x_j, s2, -((float)mx * s2)))
+ *     S   = sum_j rne(e_j * 2^23)     (integer; taken from the bit pattern of 1.0f + e_j)
+ *     y_j = rne(e_j * (127 * 2^23 / (float)S))
+ * Pins: torch.softmax on x*scale, mul(127), round (tests/test_oracle_rowops.py): the integer sum
+ * differs from the real one by less than cols * 2^-24 relative, far inside the +-1 step the
+ * comparison allows on rounding boundaries.  causal_q_len as in the HIP entry point. */
 int ti_oracle_softmax_q(const int8_t* x, int64_t x_row_stride, float scale, int8_t* y, int64_t y_row_stride,
                         int rows, int cols, int causal_q_len) {
+  if (!(scale >= 0.0f)) return -3;
+  const float s2 = scale * 1.44269504088896340736f;
 #pragma omp parallel for schedule(static)
   for (int r = 0; r < rows; ++r) {
     const int8_t* xr = x + (int64_t)r * x_row_stride;
@@ -284,11 +293,26 @@ int ti_oracle_softmax_q(const int8_t* x, int64_t x_row_stride, float scale, int8
     }
     int mx = -128;
     for (int j = 0; j < limit; ++j) if (xr[j] > mx) mx = xr[j];
-    float sum = 0.0f;
-    for (int j = 0; j < limit; ++j) sum += expf((float)(xr[j] - mx) * scale);
+    const float c = -((float)mx * s2);
+    uint64_t S = 0;
+    for (int j = 0; j < limit; ++j) {
+      const float e = exp2f(fmaf((float)xr[j], s2, c));
+      const float one_plus = 1.0f + e;
+      uint32_t bits;
+      memcpy(&bits, &one_plus, 4);
+      S += bits - 0x3f800000u;
+    }
+    const float sf = fmaf((float)(uint32_t)(S >> 24), 16777216.0f, (float)(uint32_t)(S & 0xffffffu));
+    const float rr = 1065353216.0f / sf;
     for (int j = 0; j < cols; ++j) {
-      float p = j < limit ? expf((float)(xr[j] - mx) * scale) / sum : 0.0f;
-      yr[j] = q8(p * 127.0f, 0);
+      uint32_t bits = 0;
+      if (j < limit) {
+        /* e * rr <= 127: adding 1.5 * 2^23 inside the fma rounds the exact product to the nearest
+         * integer (ties to even) and leaves it in the low byte of the sum's bit pattern */
+        const float t = fmaf(exp2f(fmaf((float)xr[j], s2, c)), rr, 12582912.0f);
+        memcpy(&bits, &t, 4);
+      }
+      yr[j] = (int8_t)(bits & 0xffu);
     }
   }
   return 0;

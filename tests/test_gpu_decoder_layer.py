@@ -97,8 +97,7 @@ def test_decoder_layer_prefill_and_decode_small():
     k2, v2 = k_old.clone(), vt_old.clone()
     trf = {}
     layer(gpu(hidden_d), kv_cache=(k2, v2), _trace=trf)
-    diff = (trf["ctx"].int() - tr["ctx"].int()).abs()
-    assert trf["scores"] is None and int((diff.amax(dim=-1) > 0).sum()) <= 1
+    assert trf["scores"] is None and torch.equal(trf["ctx"], tr["ctx"])   # the one-kernel attention is the chain, bit for bit
 
 
 def test_decoder_layer_opt13b_shapes_run():
@@ -116,18 +115,11 @@ def test_decoder_layer_opt13b_shapes_run():
     tr = {}
     out = layer(hidden.to(DEV), _trace=tr)
     assert out.shape == (1, 2048, 5120) and torch.isfinite(out).all()
-    # The two paths sum a row's exponentials in different orders.  A probability whose exact value
-    # sits within fp32 rounding of k + 0.5 can come out one step apart, and every column of that
-    # row with the same int8 score flips with it, so a rare row (measured: 1 of 81 920 here) can
-    # differ in many context values; all other rows are identical.
-    diff = (trf["ctx"].int() - tr["ctx"].int()).abs()[0].view(2048, 40, 128)
-    bad_rows = int((diff.amax(dim=-1) > 0).sum())
-    print(f"fused vs chained attention context: {bad_rows} of {2048 * 40} rows differ, max diff {int(diff.max())}")
-    assert bad_rows <= 8 and int(diff.max()) <= 16
+    # The one-kernel attention sums a row's exponentials as integers, like the stand-alone softmax
+    # kernel: same probabilities, same context, same layer output, bit for bit.
+    assert torch.equal(trf["ctx"], tr["ctx"])
     assert torch.equal(trf["q"], tr["q"]) and torch.equal(trf["vt_all"], tr["vt_all"])
-    # everything after attention works row by row: the layer outputs differ in those token rows only
-    bad_tokens = diff.amax(dim=(1, 2)) > 0
-    assert torch.equal(out_fused[0][~bad_tokens], out[0][~bad_tokens])
+    assert torch.equal(out_fused, out)
     rows = [0, 777, 2047]
     h8 = cpu(tr["h8"])[0]
     q = O.linear_a8_w8_b8_o8(h8[rows], cpu(layer.q_proj.weight), cpu(layer.q_proj.bias), np.float32(float(layer.q_proj.a)), np.float32(float(layer.q_proj.b)))
@@ -154,10 +146,7 @@ def test_decoder_layer_opt13b_shapes_run():
     trf = {}
     out_f = layer(hd.to(DEV), kv_cache=(kc2, vc2), _trace=trf)
     assert trf["scores"] is None and torch.equal(kc2, k_cache) and torch.equal(vc2, vt_cache)
-    bad_rows = int(((trf["ctx"].int() - tr["ctx"].int()).abs().view(16, 40, 128).amax(dim=-1) > 0).sum())
-    assert bad_rows <= 1
-    if bad_rows == 0:
-        assert torch.equal(out_f, out)
+    assert torch.equal(trf["ctx"], tr["ctx"]) and torch.equal(out_f, out)
 
 
 def test_layer_replayed_from_a_hip_graph_matches_eager():

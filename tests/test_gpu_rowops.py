@@ -202,13 +202,31 @@ def test_transpose_i8(rows, cols):
     assert np.array_equal(cpu(gc), want)
 
 
+def _attention_chain_checked(q, k, vt, qk_alpha, score_scale, pv_alpha, q_len):
+    """The three-launch chain on the GPU, each stage checked against the oracle applied to that
+    stage's own GPU input: scores and context bit-exact, probabilities within one step on rounding
+    boundaries.  Returns the chain's context (a device tensor)."""
+    from triton_int_amd.kernels import bmm
+    fused = _fused()
+    gq, gk, gvt = gpu(q), gpu(k), gpu(vt)
+    scores = bmm.bmm_s8t_s8n_s8t(gq, gk, qk_alpha)
+    assert np.array_equal(cpu(scores), O.bmm_s8t_s8n_s8t(q, k, np.float32(qk_alpha)))
+    probs = fused.softmax_q(scores, score_scale, causal_q_len=q_len)
+    mx, rate = mismatch_report(cpu(probs), O.softmax_q(cpu(scores), score_scale, causal_q_len=q_len))
+    assert mx <= 1 and rate <= max(2e-3, 1.5 / probs.numel()), (mx, rate)
+    ctx = bmm.bmm_s8t_s8n_s8t(probs, gvt, pv_alpha)
+    assert np.array_equal(cpu(ctx), O.bmm_s8t_s8n_s8t(cpu(probs), vt, np.float32(pv_alpha)))
+    return ctx
+
+
 @pytest.mark.parametrize("BH,S,T,q_len", [(3, 128, 128, 128), (2, 200, 336, 0), (2, 48, 272, 48), (1, 16, 2048, 16),
-                                           (2, 300, 300 + 4, 0), (4, 256, 256, 64), (1, 1, 16, 0)])
+                                           (2, 300, 300 + 4, 0), (4, 256, 256, 64), (1, 1, 16, 0), (2, 130, 4096, 0),
+                                           (3, 384, 2048, 384)])
 def test_attention_i8_against_the_three_kernel_chain(BH, S, T, q_len):
-    """Fused Q.K^T -> softmax -> P.V.  The checker is the oracle's chain of the three steps.  The
-    int8 scores inside the kernel are the BMM's bit for bit, so differences can only come from
-    probabilities that sit on a rounding boundary (allowed: one step, rarely) and what they do to a
-    context value (one step)."""
+    """Fused Q.K^T -> softmax -> P.V.  Its int8 scores are the BMM's and its probabilities the softmax
+    kernel's bit for bit (a row's exponentials are summed as integers, so the order in which the
+    kernels visit the keys does not matter): the context must EQUAL the three-launch chain's, whose
+    stages are checked against the oracle one by one."""
     fused = _fused()
     T = (T + 15) // 16 * 16
     g = rng(BH * 1000 + S + T)
@@ -217,14 +235,11 @@ def test_attention_i8_against_the_three_kernel_chain(BH, S, T, q_len):
     k = g.integers(-127, 128, size=(BH, T, D), dtype=np.int8)
     vt = g.integers(-127, 128, size=(BH, D, T), dtype=np.int8)
     seen_nontrivial = False
-    for qk_alpha, score_scale, pv_alpha in ((1e-3, 0.05, 1.0 / 127.0), (4e-3, 0.02, 0.03)):
-        want = O.attention_i8(q, k, vt, qk_alpha, score_scale, pv_alpha, causal_q_len=q_len)
-        got = cpu(fused.attention_i8(gpu(q), gpu(k), gpu(vt), qk_alpha, score_scale, pv_alpha, causal_q_len=q_len))
-        mx, rate = mismatch_report(got, want)
-        print(f"attention_i8 BH {BH} S {S} T {T} q_len {q_len} alpha {qk_alpha}: max diff {mx}, mismatch rate {rate:.2e}")
-        bad_rows = int((np.abs(got.astype(int) - want.astype(int)).max(axis=-1) > 0).sum())
-        assert got.shape == (BH, S, D) and bad_rows <= max(1, BH * S // 1000), f"{bad_rows} rows differ (max {mx})"
-        seen_nontrivial = seen_nontrivial or np.unique(got).size > 8
+    for qk_alpha, score_scale, pv_alpha in ((1e-3, 0.05, 1.0 / 127.0), (4e-3, 0.02, 0.03), (-2e-3, 0.5, 0.02)):
+        want = _attention_chain_checked(q, k, vt, qk_alpha, score_scale, pv_alpha, q_len)
+        got = fused.attention_i8(gpu(q), gpu(k), gpu(vt), qk_alpha, score_scale, pv_alpha, causal_q_len=q_len)
+        assert got.shape == (BH, S, D) and torch.equal(got, want), f"alpha {qk_alpha} scale {score_scale}: {int((got != want).sum())} values differ"
+        seen_nontrivial = seen_nontrivial or np.unique(cpu(got)).size > 8
     assert seen_nontrivial or T >= 1024  # long rows of random scores spread the probabilities below 1/254
 
 
@@ -233,23 +248,18 @@ def test_attention_i8_against_the_three_kernel_chain(BH, S, T, q_len):
                                            (2, 12, 48, 4)])
 def test_attention_i8_few_query_rows(BH, S, T, q_len):
     """16 or fewer query rows per head (decode, short chunks) run the one-workgroup-per-head kernel:
-    same checker and same bar as above.  Its exponent is taken against the row maximum like the
-    stand-alone softmax kernel's, so only the order of a row's sum differs from the chain."""
+    same checker and same bar as above: equal to the chain."""
     fused = _fused()
     g = rng(BH * 77 + S * 5 + T)
     D = 128
     q = g.integers(-127, 128, size=(BH, S, D), dtype=np.int8)
     k = g.integers(-127, 128, size=(BH, T, D), dtype=np.int8)
     vt = g.integers(-127, 128, size=(BH, D, T), dtype=np.int8)
-    for qk_alpha, score_scale, pv_alpha in ((1e-3, 0.05, 1.0 / 127.0), (4e-3, 0.02, 0.03), (2e-3, 0.3, 0.02)):
-        want = O.attention_i8(q, k, vt, qk_alpha, score_scale, pv_alpha, causal_q_len=q_len)
+    for qk_alpha, score_scale, pv_alpha in ((1e-3, 0.05, 1.0 / 127.0), (4e-3, 0.02, 0.03), (2e-3, 0.3, 0.02), (3e-3, 1.5, 0.02)):
+        want = _attention_chain_checked(q, k, vt, qk_alpha, score_scale, pv_alpha, q_len)
         out = torch.full((BH, S, D), 77, dtype=torch.int8, device=DEV)
         fused.attention_i8(gpu(q), gpu(k), gpu(vt), qk_alpha, score_scale, pv_alpha, causal_q_len=q_len, out=out)
-        got = cpu(out)
-        mx, rate = mismatch_report(got, want)
-        bad_rows = int((np.abs(got.astype(int) - want.astype(int)).max(axis=-1) > 0).sum())
-        print(f"attention_i8 (few rows) BH {BH} S {S} T {T} q_len {q_len} scale {score_scale}: max diff {mx}, rows {bad_rows}")
-        assert bad_rows <= max(1, BH * S // 200), f"{bad_rows} rows differ (max {mx})"
+        assert torch.equal(out, want), f"scale {score_scale}: {int((out != want).sum())} values differ"
 
 
 def test_attention_i8_strided_views_and_errors():
@@ -275,8 +285,10 @@ def test_attention_i8_strided_views_and_errors():
     assert mx <= 1 and rate < 5e-3
     with pytest.raises(AssertionError):  # head dimension other than 128
         fused.attention_i8(gpu(q3[:, :, :64].copy()), gpu(k3[:, :, :64].copy()), gpu(vt[:, :64].copy()), 1e-3, 0.05, 0.01)
-    with pytest.raises(AssertionError):  # score scale too large for the fixed-bound exponent
-        fused.attention_i8(gq, gk, gvt, 1e-3, 0.5, 0.01)
+    with pytest.raises(AssertionError):  # the exponent is taken against the row's largest score: the scale must be positive
+        fused.attention_i8(gq, gk, gvt, 1e-3, -0.5, 0.01)
+    with pytest.raises(AssertionError):
+        fused.softmax_q(gpu(np.zeros((4, 32), np.int8)), -0.1)
 
 
 @pytest.mark.parametrize("rows,cols", [(2048, 5120), (37, 300), (5, 1), (3, 8193), (64, 768), (9, 20480), (2, 40000)])

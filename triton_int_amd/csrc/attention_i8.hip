@@ -8,18 +8,17 @@
 // At 2048 x 2048 scores per head the two intermediates are 4 x 168 MB of HBM traffic for 40 heads.
 // This kernel computes the same three steps per 32 x 32 block of scores in registers: the int8
 // score quantisation, the probability quantisation and the context quantisation are the same
-// fp32 operations as in the three kernels; only the order in which a row's exponentials are
-// summed differs (and the exponent is taken against the fixed bound 127 instead of the row
-// maximum, which cancels in the quotient), so a probability can differ by one step when
-// 127 * e / sum falls within rounding error of a half; every column of that row with the same
-// int8 score then flips with it, and the row's context values can move by a few steps (measured:
-// 1 row of 81 920 at 2048 keys; all other rows bit-identical to the three-kernel chain).
+// fp32 operations as in the three kernels, and a row's exponentials are summed as integers (see
+// the softmax-quantise arithmetic in ti_common.h), so the result is the three-kernel chain's bit
+// for bit although the keys are visited in another order.
 //
-// Two passes over the keys of a query block, as the probabilities need the whole row's sum before
-// they can be quantised: pass 1 computes scores and sums exponentials, pass 2 recomputes the
-// scores (K = 128 deep: cheap), forms the int8 probabilities in the MFMA operand layout straight
-// from the accumulator registers (two half-wave swaps put a row's keys in order) and feeds them
-// to the P.V MFMAs, so P never goes through memory.
+// Three passes over the keys of a query block.  Pass 0 finds each row's largest score (the
+// exponent's reference point): the quantisation is monotone in the int32 accumulator, so it is a
+// maximum over accumulators, one instruction per two scores.  Pass 1 recomputes the scores
+// (K = 128 deep: cheap) and sums the exponentials.  Pass 2 recomputes them once more, forms the
+// int8 probabilities in the MFMA operand layout straight from the accumulator registers (two
+// half-wave swaps put a row's keys in order) and feeds them to the P.V MFMAs, so P never goes
+// through memory.
 //
 // (Blocks of 16 or fewer query rows take attention_decode_i8_kernel further down instead.)
 //
@@ -135,7 +134,69 @@ __global__ __launch_bounds__(256, 2) void attention_i8_kernel(AttnParams p) {
   };
 
   const float MAGIC = 12582912.0f;  // 1.5 * 2^23: adding it rounds to the nearest even integer
-  const float c127 = -(127.0f * p.s2);
+
+  // ================= pass 0: each row's largest score =================
+  // q8(alpha * f(acc)) does not decrease with acc when alpha >= 0 (and does not increase when
+  // alpha < 0), so the largest score is the quantised largest (smallest) accumulator.
+  const bool want_max = p.qk_alpha >= 0.0f;
+  int ext = want_max ? (int)0x80000000 : 0x7fffffff;
+  auto score_ext_t = [&](const char* kt, int key0, auto mask_tag, auto max_tag) {
+    constexpr bool MASK = decltype(mask_tag)::value;
+    constexpr bool MAX = decltype(max_tag)::value;
+    v4i kf[2][4];
+#pragma unroll
+    for (int ds = 0; ds < 4; ++ds)
+#pragma unroll
+      for (int b = 0; b < 2; ++b) kf[b][ds] = *(const v4i*)(kt + (b * 32 + lrow) * AT_KP + ds * 32 + lhi * 16);
+    v16i s[2];
+    const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int ds = 0; ds < 4; ++ds)
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+        s[b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[b][ds], qf[ds], ds == 0 ? zero : s[b], 0, 0, 0);
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        int v = s[b][r];
+        if constexpr (MASK) {
+          const int key = key0 + 32 * b + 8 * (r >> 2) + 4 * lhi + (r & 3);
+          v = key < lim_lane ? v : (MAX ? (int)0x80000000 : 0x7fffffff);
+        }
+        ext = MAX ? max(ext, v) : min(ext, v);
+      }
+  };
+  auto score_ext = [&](const char* kt, int key0) {
+    const bool mask = key0 + AT_KT > lim_lo;
+    if (want_max) {
+      if (mask) score_ext_t(kt, key0, std::true_type{}, std::true_type{});
+      else score_ext_t(kt, key0, std::false_type{}, std::true_type{});
+    } else {
+      if (mask) score_ext_t(kt, key0, std::true_type{}, std::false_type{});
+      else score_ext_t(kt, key0, std::false_type{}, std::false_type{});
+    }
+  };
+  fetch(0, false);
+  stash(0, false);
+  __syncthreads();
+  for (int t = 0; t < ntiles; ++t) {
+    if (t + 1 < ntiles) fetch(t + 1, false);
+    const char* kt = lds + (t & 1) * (AT_KBYTES + AT_VBYTES);
+    if (wave_live && t * AT_KT < lim_hi) score_ext(kt, t * AT_KT);
+    if (t + 1 < ntiles) stash((t + 1) & 1, false);
+    __syncthreads();
+  }
+  {
+    const int other = __shfl_xor(ext, 32, 64);  // the two lane halves hold different keys of the same row
+    ext = want_max ? max(ext, other) : min(ext, other);
+  }
+  float cref;  // -(largest score * s2): the exponent's reference point of this lane's row
+  {
+    float v = (float)ext * p.qk_alpha;
+    v = __builtin_amdgcn_fmed3f(v, -128.0f, 127.0f);
+    cref = -(__builtin_rintf(v) * p.s2);
+  }
   // Scores of one 64-key tile -> exponentials.  The tile's two 32-key blocks are two independent
   // MFMA chains, interleaved, with all fragment reads issued first; e[b][r] belongs to key
   // key0 + 32*b + 8*(r/4) + 4*lhi + r%4.  A block that lies wholly beyond the wave's last visible
@@ -148,15 +209,12 @@ __global__ __launch_bounds__(256, 2) void attention_i8_kernel(AttnParams p) {
 #pragma unroll
       for (int b = 0; b < 2; ++b) kf[b][ds] = *(const v4i*)(kt + (b * 32 + lrow) * AT_KP + ds * 32 + lhi * 16);
     v16i s[2];
-#pragma unroll
-    for (int b = 0; b < 2; ++b)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) s[b][r] = 0;
+    const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
     for (int ds = 0; ds < 4; ++ds)
 #pragma unroll
       for (int b = 0; b < 2; ++b)
-        s[b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[b][ds], qf[ds], s[b], 0, 0, 0);  // rows of the result = keys
+        s[b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[b][ds], qf[ds], ds == 0 ? zero : s[b], 0, 0, 0);  // rows of the result = keys
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
 #pragma unroll
@@ -164,7 +222,7 @@ __global__ __launch_bounds__(256, 2) void attention_i8_kernel(AttnParams p) {
         float v = (float)s[b][r] * p.qk_alpha;
         v = __builtin_amdgcn_fmed3f(v, -128.0f, 127.0f);
         const float x = __builtin_rintf(v);  // the int8 score, as a float (round half to even, like the BMM's)
-        e[b][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x, p.s2, c127));
+        e[b][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(x, p.s2, cref));
       }
       if constexpr (MASK) {
 #pragma unroll
@@ -183,8 +241,8 @@ __global__ __launch_bounds__(256, 2) void attention_i8_kernel(AttnParams p) {
     else score_exp_t(kt, key0, e, std::false_type{});
   };
 
-  // ================= pass 1: row sums =================
-  float sum = 0.0f;
+  // ================= pass 1: row sums (exact integers, see ti_common.h) =================
+  unsigned long long sum = 0;
   fetch(0, false);
   stash(0, false);
   __syncthreads();
@@ -194,19 +252,24 @@ __global__ __launch_bounds__(256, 2) void attention_i8_kernel(AttnParams p) {
     if (wave_live && t * AT_KT < lim_hi) {
       float e[2][16];
       score_exp(kt, t * AT_KT, e);
-      float s0 = 0.0f, s1 = 0.0f;
+      unsigned s0 = 0, s1 = 0;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        s0 += e[0][r];
-        s1 += e[1][r];
+        s0 += sm_unit_bits(e[0][r]);
+        s1 += sm_unit_bits(e[1][r]);
       }
-      sum += s0 + s1;
+      sum += (unsigned)(s0 + s1 - 32u * SM_ONE_BITS);  // modulo 2^32: the tile's 32 units of this lane, below 2^29
     }
     if (t + 1 < ntiles) stash((t + 1) & 1, false);
     __syncthreads();
   }
-  sum += __shfl_xor(sum, 32, 64);  // the two lane halves hold different keys of the same row
-  const float rinv = 127.0f / sum;
+  {
+    // the two lane halves hold different keys of the same row
+    const unsigned lo = (unsigned)__shfl_xor((int)(unsigned)sum, 32, 64);
+    const unsigned hi = (unsigned)__shfl_xor((int)(unsigned)(sum >> 32), 32, 64);
+    sum += ((unsigned long long)hi << 32) | lo;
+  }
+  const float rinv = sm_scale_from_sum(sum);
 
   // ================= pass 2: probabilities and P.V =================
   v16i o[4];
@@ -314,7 +377,7 @@ __global__ __launch_bounds__(AD_WAVES * 64) void attention_decode_i8_kernel(Attn
   constexpr int HOIST = CPW >= 16 ? (GPW < 4 ? GPW : 4) : GPW;  // V^T operands fetched before the softmax reductions
   __shared__ __attribute__((aligned(16))) char p_lds[16 * PP];
   __shared__ float red_max[AD_WAVES][16];
-  __shared__ float red_sum[AD_WAVES][16];
+  __shared__ unsigned red_sum[AD_WAVES][16];
   __shared__ __attribute__((aligned(16))) v4i ctx_red[AD_WAVES][64];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -335,7 +398,7 @@ __global__ __launch_bounds__(AD_WAVES * 64) void attention_decode_i8_kernel(Attn
   const int NG = (p.T + 63) >> 6;   // 64-key groups
   const int db = dbase + wave % DBW, kh = wave / DBW;
 
-  // ---- scores: f = int8 score + 128 as a float, -inf where masked or beyond T
+  // ---- scores: f = the int8 score as a float, -inf where masked or beyond T
   v4i qf[2];
 #pragma unroll
   for (int ks = 0; ks < 2; ++ks)
@@ -366,7 +429,7 @@ __global__ __launch_bounds__(AD_WAVES * 64) void attention_decode_i8_kernel(Attn
         float v = (float)acc[r] * p.qk_alpha;
         v = __builtin_amdgcn_fmed3f(v, -128.0f, 127.0f);
         const int key = c * 16 + 4 * kq + r;
-        f[b0 + i][r] = key < limit ? __builtin_rintf(v) + 128.0f : NEG;
+        f[b0 + i][r] = key < limit ? __builtin_rintf(v) : NEG;
       }
     }
   }
@@ -390,22 +453,25 @@ __global__ __launch_bounds__(AD_WAVES * 64) void attention_decode_i8_kernel(Attn
 #pragma unroll
   for (int w = 0; w < AD_WAVES; ++w) mx = fmaxf(mx, red_max[w][n]);
   const float c0 = -(mx * p.s2);
-  float sum = 0.0f;
+  // exact integer row sum (see ti_common.h): a lane holds at most 64 scores (below 2^29 units), the
+  // four lanes of a query below 2^31, the 16 waves meet in 64 bits
+  unsigned bits = 0;
 #pragma unroll
   for (int i = 0; i < CPW; ++i)
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       f[i][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(f[i][r], p.s2, c0));
-      sum += f[i][r];
+      bits += sm_unit_bits(f[i][r]);
     }
-  sum += __shfl_xor(sum, 16, 64);
-  sum += __shfl_xor(sum, 32, 64);
-  if (kq == 0) red_sum[wave][n] = sum;
+  bits -= (unsigned)(CPW * 4) * SM_ONE_BITS;  // modulo 2^32
+  bits += (unsigned)__shfl_xor((int)bits, 16, 64);
+  bits += (unsigned)__shfl_xor((int)bits, 32, 64);
+  if (kq == 0) red_sum[wave][n] = bits;
   __syncthreads();
-  sum = 0.0f;
+  unsigned long long sum = 0;
 #pragma unroll
   for (int w = 0; w < AD_WAVES; ++w) sum += red_sum[w][n];
-  const float rcp = 127.0f / sum;
+  const float rcp = sm_scale_from_sum(sum);
 
   // ---- int8 probabilities into LDS, key order; keys in [T, 64 * NG) get zeros (their f is -inf)
 #pragma unroll
@@ -484,8 +550,8 @@ extern "C" int ti_attention_i8(const int8_t* q, int64_t q_batch_stride, int64_t 
   // exponentials are taken against the largest possible score (127): the smallest one must stay a
   // normal fp32 number
   const float s2 = score_scale * 1.44269504088896340736f;
-  if (!(score_scale > 0.0f) || s2 * 255.0f > 120.0f)
-    return fail(TI_E_COMBO, "score_scale %g outside (0, 0.32]: use the three-kernel path", (double)score_scale);
+  if (!(score_scale > 0.0f) || !(s2 < 3.0e38f))
+    return fail(TI_E_COMBO, "score_scale %g is not a positive finite number", (double)score_scale);
   const int64_t lim32 = (int64_t)1 << 31;
   const bool few_rows = S <= 16 && T <= AD_MAXT && (int64_t)T * k_row_stride < lim32 && (int64_t)AT_D * vt_row_stride < lim32 &&
                         (int64_t)S * q_row_stride < lim32;

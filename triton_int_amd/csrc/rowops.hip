@@ -269,6 +269,17 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// exact sum over the 64 lanes of values below 2^31: the low and high 16 bits are summed separately
+__device__ __forceinline__ unsigned long long wave_sum_u64(unsigned v) {
+  unsigned lo = v & 0xffffu, hi = v >> 16;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    lo += (unsigned)__shfl_xor((int)lo, off, 64);
+    hi += (unsigned)__shfl_xor((int)hi, off, 64);
+  }
+  return ((unsigned long long)hi << 16) + lo;
+}
+
 // Rows whose start and length are multiples of 16 bytes.  Every load of a row is issued before the
 // first use: buffer loads whose offset is pushed out of range for chunks beyond the causal limit
 // (they return 0 without touching memory), then masking in registers.  Stores are range-checked
@@ -302,12 +313,11 @@ __global__ __launch_bounds__(SM_WAVES * 64) void softmax_q_kernel(const int8_t* 
     if (c0 >= limit) continue;  // whole 1 KB pieces beyond the limit cost no VALU work
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      const unsigned u = (unsigned)w[j][g] ^ 0x80808080u;
-      // the compiler turns these into v_cvt_f32_ubyte0..3
-      f[j][4 * g + 0] = (float)(u & 0xffu);
-      f[j][4 * g + 1] = (float)((u >> 8) & 0xffu);
-      f[j][4 * g + 2] = (float)((u >> 16) & 0xffu);
-      f[j][4 * g + 3] = (float)(u >> 24);
+      const unsigned u = (unsigned)w[j][g];
+      f[j][4 * g + 0] = sbyte_to_float<0>(u);
+      f[j][4 * g + 1] = sbyte_to_float<1>(u);
+      f[j][4 * g + 2] = sbyte_to_float<2>(u);
+      f[j][4 * g + 3] = sbyte_to_float<3>(u);
     }
     if (c0 + 16 > limit) {  // the chunk that straddles the limit
 #pragma unroll
@@ -319,7 +329,8 @@ __global__ __launch_bounds__(SM_WAVES * 64) void softmax_q_kernel(const int8_t* 
   mx = wave_max(mx);
   const float s2 = scale * 1.44269504088896340736f;  // exp(v) = exp2(v * log2 e)
   const float c = -(mx * s2);
-  float sum = 0.0f;
+  // exponentials and their exact integer sum (see ti_common.h); a lane's partial sum stays below 2^31
+  unsigned bits = 0;
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
     const int c0 = (j * 64 + lane) * 16;
@@ -327,11 +338,11 @@ __global__ __launch_bounds__(SM_WAVES * 64) void softmax_q_kernel(const int8_t* 
 #pragma unroll
     for (int t = 0; t < 16; ++t) {
       f[j][t] = __builtin_amdgcn_exp2f(__builtin_fmaf(f[j][t], s2, c));
-      sum += f[j][t];
+      bits += sm_unit_bits(f[j][t]);
     }
+    bits -= 16u * SM_ONE_BITS;  // modulo 2^32, like the additions: what is left is the chunk's sum of u
   }
-  sum = wave_sum(sum);
-  const float r = 127.0f / sum;
+  const float r = sm_scale_from_sum(wave_sum_u64(bits));
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
     const int c0 = (j * 64 + lane) * 16;
@@ -349,12 +360,6 @@ __global__ __launch_bounds__(SM_WAVES * 64) void softmax_q_kernel(const int8_t* 
     __builtin_amdgcn_raw_buffer_store_b128(o, ry, c0, 0, 2);  // dropped beyond the row's end
   }
 }
-
-// Per element the work is: byte -> float (v_cvt_f32_ubyteN on the sign-flipped dword, so the float
-// is x + 128), one fma that forms (x - max) * scale * log2(e), the hardware exp2, one add for the
-// sum; then one fma e * (127 / sum) + 1.5 * 2^23, whose low byte is the rounded probability (it
-// lies in [0, 127], no clamp), and byte permutes to pack.  16-byte chunks that lie wholly beyond a
-// causal limit are neither read nor computed, the one chunk that straddles it is masked.
 template <int VPT>
 __global__ __launch_bounds__(SM_WAVES * 64) void softmax_q_any_kernel(const int8_t* __restrict__ x, int64_t x_rs,
                                                                   float scale, int8_t* __restrict__ y, int64_t y_rs,
@@ -366,9 +371,9 @@ __global__ __launch_bounds__(SM_WAVES * 64) void softmax_q_any_kernel(const int8
   const int8_t* xr = x + (int64_t)row * x_rs;
   int8_t* yr = y + (int64_t)row * y_rs;
   const bool vec = ((((uintptr_t)xr) | ((uintptr_t)yr)) & 15) == 0;
-  const float NEG = -1.0f;  // below every x + 128 >= 0: excluded from the maximum, flags a masked element
+  const float NEG = -__builtin_inff();  // drops out of the maximum; its exponential is 0 (scale > 0) or masked below
 
-  // f[j][t] = x + 128 as a float, or NEG for masked / out-of-row elements
+  // f[j][t] = the score as a float, or NEG for masked / out-of-row elements
   float f[VPT][16];
   float mx = NEG;
 #pragma unroll
@@ -383,12 +388,10 @@ __global__ __launch_bounds__(SM_WAVES * 64) void softmax_q_any_kernel(const int8
       v4u w = __builtin_nontemporal_load((const v4u*)(xr + c0));
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const unsigned u = w[g] ^ 0x80808080u;
-        // the compiler turns these into v_cvt_f32_ubyte0..3
-        f[j][4 * g + 0] = (float)(u & 0xffu);
-        f[j][4 * g + 1] = (float)((u >> 8) & 0xffu);
-        f[j][4 * g + 2] = (float)((u >> 16) & 0xffu);
-        f[j][4 * g + 3] = (float)(u >> 24);
+        f[j][4 * g + 0] = sbyte_to_float<0>(w[g]);
+        f[j][4 * g + 1] = sbyte_to_float<1>(w[g]);
+        f[j][4 * g + 2] = sbyte_to_float<2>(w[g]);
+        f[j][4 * g + 3] = sbyte_to_float<3>(w[g]);
       }
       if (c0 + 16 > limit) {
 #pragma unroll
@@ -399,7 +402,7 @@ __global__ __launch_bounds__(SM_WAVES * 64) void softmax_q_any_kernel(const int8
     } else {
 #pragma unroll
       for (int t = 0; t < 16; ++t) {
-        f[j][t] = c0 + t < limit ? (float)((int)xr[c0 + t] + 128) : NEG;
+        f[j][t] = c0 + t < limit ? (float)(int)xr[c0 + t] : NEG;
         mx = fmaxf(mx, f[j][t]);
       }
     }
@@ -407,22 +410,22 @@ __global__ __launch_bounds__(SM_WAVES * 64) void softmax_q_any_kernel(const int8
   mx = wave_max(mx);
   const float s2 = scale * 1.44269504088896340736f;  // exp(v) = exp2(v * log2 e)
   const float c = -(mx * s2);
-  float sum = 0.0f;
+  unsigned bits = 0;
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
     const int c0 = (j * 64 + lane) * 16;
     if (c0 >= limit) continue;
 #pragma unroll
     for (int t = 0; t < 16; ++t) f[j][t] = __builtin_amdgcn_exp2f(__builtin_fmaf(f[j][t], s2, c));
-    if (c0 + 16 > limit) {  // the chunk that straddles the limit (or the end of the row)
+    if (c0 + 16 > limit) {  // the chunk that straddles the limit (or the end of the row): with scale 0 its NEG elements gave NaN
 #pragma unroll
       for (int t = 0; t < 16; ++t) f[j][t] = c0 + t < limit ? f[j][t] : 0.0f;
     }
 #pragma unroll
-    for (int t = 0; t < 16; ++t) sum += f[j][t];
+    for (int t = 0; t < 16; ++t) bits += sm_unit_bits(f[j][t]);
+    bits -= 16u * SM_ONE_BITS;
   }
-  sum = wave_sum(sum);
-  const float r = 127.0f / sum;
+  const float r = sm_scale_from_sum(wave_sum_u64(bits));
 #pragma unroll
   for (int j = 0; j < VPT; ++j) {
     const int c0 = (j * 64 + lane) * 16;
@@ -634,6 +637,7 @@ int ti_softmax_q(const int8_t* x, int64_t x_row_stride, float scale, int8_t* y, 
   if (causal_q_len > cols) return ti::fail(TI_E_SHAPE, "causal_q_len %d > cols %d", causal_q_len, cols);
   if (causal_q_len > 0 && rows % causal_q_len) return ti::fail(TI_E_SHAPE, "rows %d not a multiple of causal_q_len %d", rows, causal_q_len);
   if (cols > 64 * 16 * 8) return ti::fail(TI_E_SHAPE, "softmax rows longer than 8192 are not supported");
+  if (!(scale >= 0.0f)) return ti::fail(TI_E_COMBO, "the score scale must be >= 0 (the exponent is taken against the row's largest score)");
   int rc = ti::check_device();
   if (rc != TI_OK) return rc;
   hipStream_t s = (hipStream_t)stream;

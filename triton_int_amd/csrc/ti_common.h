@@ -64,6 +64,40 @@ __device__ __forceinline__ float gelu_tanh_scaled(float x, float scale) {
   return (x * (1.0f - r)) * scale;
 }
 
+// ---- softmax-quantise arithmetic -----------------------------------------------------------------
+// int8 scores x -> int8 probabilities rne(127 * softmax(x * scale)) the same way in every kernel that
+// forms them (the stand-alone softmax kernels and both attention kernels), so that their results
+// agree bit for bit whatever the order in which they visit a row:
+//   mx  = the row's largest visible score (an integer: exact in any order)
+//   t   = fma(float(x), s2, c),  c = -(float(mx) * s2),  s2 = scale * log2(e)
+//   e   = exp2(t)                                      (in (0, 1], exactly 1 at the maximum)
+//   u   = rne(e * 2^23), taken from the bit pattern of 1.0f + e
+//   S   = sum of u over the row: an integer, so any order and any grouping give the same S
+//   r   = 127 * 2^23 / float(S)                        (float(S) correctly rounded, IEEE division)
+//   p   = rne(e * r): the low byte of the bit pattern of fma(e, r, 1.5 * 2^23)
+constexpr unsigned SM_ONE_BITS = 0x3f800000u;  // bit pattern of 1.0f: sm_unit_bits(e) - SM_ONE_BITS = u
+
+__device__ __forceinline__ unsigned sm_unit_bits(float e) { return __float_as_uint(1.0f + e); }
+
+// 127 * 2^23 / S for the exact row sum S (< 2^48)
+__device__ __forceinline__ float sm_scale_from_sum(unsigned long long S) {
+  const float hi = (float)(unsigned)(S >> 24), lo = (float)(unsigned)(S & 0xffffffu);  // both exact
+  const float sf = __builtin_fmaf(hi, 16777216.0f, lo);                                // rounded once
+  return 1065353216.0f / sf;
+}
+
+// byte n (0..3) of w as a signed int8, converted to float: one instruction (sub-dword source select
+// with sign extension)
+template <int N>
+__device__ __forceinline__ float sbyte_to_float(unsigned w) {
+  float f;
+  if constexpr (N == 0) asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_0" : "=v"(f) : "v"(w));
+  else if constexpr (N == 1) asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1" : "=v"(f) : "v"(w));
+  else if constexpr (N == 2) asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_2" : "=v"(f) : "v"(w));
+  else asm("v_cvt_f32_i32_sdwa %0, sext(%1) dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_3" : "=v"(f) : "v"(w));
+  return f;
+}
+
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
   __bf16 h = (__bf16)f;  // v_cvt_pk_bf16_f32, round-to-nearest-even
   return __builtin_bit_cast(uint16_t, h);

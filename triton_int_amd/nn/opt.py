@@ -159,7 +159,7 @@ class W8A8OPTDecoderLayer(torch.nn.Module):
         ctx = torch.empty((B, S, H), dtype=torch.int8, device=hidden.device)
         # 16 or fewer query rows (decode) against up to 4096 keys run the kernel's one-workgroup-per-head form
         fused = (self.fused_attention and (S >= self.fused_attention_min_queries or (S <= 16 and T <= 4096))
-                 and self.head_dim == 128 and T % 16 == 0 and 0.0 < self.score_scale <= 0.32)
+                 and self.head_dim == 128 and T % 16 == 0 and self.score_scale > 0.0)
         scores = probs = None
         if fused:
             for b in range(B):
