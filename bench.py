@@ -29,6 +29,12 @@ METRIC = "int8 GEMM TOPS (% MFMA peak), LN/GELU GB/s, W8A8 OPT-13B layer ms"
 MEASURED_TRAFFIC_BYTES = {
     "ws_256x128x128_w2x2_s1_p3_l4/int8": (2.0 * 52601 + 1.0 * 15384) * 1024,
 }
+# where that reading comes from: the summary file and what the kernel's tile order was when it was
+# taken (the figure is only as fresh as that file; bench.py does not re-measure it)
+MEASURED_TRAFFIC_SOURCE = {
+    "ws_256x128x128_w2x2_s1_p3_l4/int8": "profiles/gemm_ws_opt67b_linear_set_counters.md (FETCH_SIZE x2.0 + WRITE_SIZE x1.0, KiB per "
+                                         "dispatch averaged over the 5 launches of a step)",
+}
 INT8_PEAK_TOPS = 5000.0   # MI355X dense INT8 MFMA, published
 HBM_PEAK_GBPS = 8000.0    # MI355X HBM3E, published
 
@@ -321,6 +327,85 @@ def extras(torch, dev):
     return out
 
 
+def m_sweep(torch, dev, N, K, lib):
+    """The reference's own benchmark (kernels/linear.py:960-1070): int8 x int8 -> fp32 linear with an
+    fp32 bias over M, weights [N, K]; operands made like the reference's (`randn(fp16).to(int8)`),
+    per-launch event timing, quantiles 0.5 / 0.2 / 0.8 as its `do_bench(quantiles=...)` call."""
+    from triton_int_amd.kernels import linear
+
+    out = {}
+    b = torch.randn((N, K), device=dev, dtype=torch.float16).to(torch.int8)
+    bias = torch.randn(N, device=dev)
+    one = torch.tensor(1.0, device=dev)
+    for M in (32, 64, 128, 256, 1024, 2048, 4096, 8192, 16384):
+        a = torch.randn((M, K), device=dev, dtype=torch.float16).to(torch.int8)
+        for _ in range(3):
+            linear.linear_a8_w8_bfp32_ofp32(a, b, bias, one, one)
+        reps = 20
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+        for s_, e_ in ev:
+            s_.record()
+            linear.linear_a8_w8_bfp32_ofp32(a, b, bias, one, one)
+            e_.record()
+        torch.cuda.synchronize()
+        ts = sorted(s_.elapsed_time(e_) for s_, e_ in ev)
+        p50 = ts[len(ts) // 2]
+        out[f"M{M}"] = {"ms_p50_p20_p80": [p50, ts[len(ts) // 5], ts[4 * len(ts) // 5]],
+                        "TOPS": 2.0 * M * N * K / p50 / 1e9,
+                        "kernel": lib.ti_gemm_config_name(lib.ti_gemm_last_config()).decode(),
+                        "k_splits": lib.ti_gemm_last_splits()}
+    return out
+
+
+def cpu_baseline_rows(torch, budget_s=4.0):
+    """CPU emulation (torch on the host cores) of the HBM-bound kernels on bounded samples of their
+    benchmark shapes: dq + add + LayerNormQ (functional/fused.py:6-15), GELU-quant, one head of Q.K^T."""
+    import torch.nn.functional as F
+
+    from oracle import cpu_emulation as E
+
+    torch.set_num_threads(min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16"))))
+    g = torch.Generator().manual_seed(7)
+    out = {"cores": torch.get_num_threads()}
+
+    def timed(fn, unit_bytes, what):
+        fn()
+        n, t0 = 0, time.perf_counter()
+        while time.perf_counter() - t0 < budget_s / 3 or n == 0:
+            fn()
+            n += 1
+        el = (time.perf_counter() - t0) / n
+        return {"GBps": unit_bytes / el / 1e9, "ms": el * 1e3, "sample": what}
+
+    rows, cols = 1024, 5120
+    acc = torch.randint(-2**20, 2**20 + 1, (rows, cols), dtype=torch.int32, generator=g)
+    res, gam, bet = torch.randn((rows, cols), generator=g), torch.randn(cols, generator=g) * 2 + 20, torch.randn(cols, generator=g) * 2
+    out["dq_add_layernorm_q"] = timed(lambda: E.dq_add_layernorm_q(acc, 1e-5, res, gam, bet, 1e-5), rows * cols * 13,
+                                      f"{rows} of 8192 rows x {cols}")
+    xg = torch.randn((512, 20480), generator=g)
+    out["gelu_q"] = timed(lambda: torch.clamp(torch.round(F.gelu(xg, approximate="tanh") * 20.0), -128, 127).to(torch.int8),
+                          xg.numel() * 5, "512 of 8192 rows x 20480")
+    q = torch.randint(-127, 128, (1, 512, 128), dtype=torch.int8, generator=g)
+    k = torch.randint(-127, 128, (1, 2048, 128), dtype=torch.int8, generator=g)
+    r = timed(lambda: E.bmm_o8(q, k, 1e-3), 512 * 128 + 2048 * 128 + 512 * 2048, "512 query rows of one of 160 heads, 2048 keys")
+    r["TOPS"] = 2.0 * 512 * 2048 * 128 / (r["ms"] * 1e-3) / 1e12
+    out["bmm_qk_s8"] = r
+    return out
+
+
+def attention_mismatch(torch, dev):
+    """The one-kernel attention against the BMM -> softmax -> BMM chain on the layer's shape (40 heads,
+    2048 x 2048, causal): rows of the context that differ and the largest difference."""
+    from triton_int_amd.kernels import bmm, fused
+
+    q, k = (torch.randint(-127, 128, (40, 2048, 128), dtype=torch.int8, device=dev) for _ in range(2))
+    vt = torch.randint(-127, 128, (40, 128, 2048), dtype=torch.int8, device=dev)
+    one = fused.attention_i8(q, k, vt, 1e-3, 0.05, 1.0 / 127.0, causal_q_len=2048)
+    chain = bmm.bmm_s8t_s8n_s8t(fused.softmax_q(bmm.bmm_s8t_s8n_s8t(q, k, 1e-3), 0.05, causal_q_len=2048), vt, 1.0 / 127.0)
+    d = (one.int() - chain.int()).abs()
+    return {"rows": 40 * 2048, "rows_differing": int((d.amax(dim=-1) > 0).sum()), "max_step": int(d.max())}
+
+
 def decoder_layer_ms(torch, dev):
     """W8A8 OPT-13B-shaped decoder layer (hidden 5120, 40 heads, FFN 20480), random int8 weights:
     prefill (batch 1, seq 2048) and decode (16 tokens against a 2048-long int8 KV).  Two layers with
@@ -449,6 +534,9 @@ def main():
         torch.cuda.synchronize()
         return
     layers = build_linear_set(torch, dev)
+    # a second set of weights and activations (other seed): the timed steps alternate between the two,
+    # 2 x 264 MB of operands, so that no step finds its operands in the 256 MB Infinity Cache
+    layers_b = build_linear_set(torch, dev, seed=4321)
     # which kernel does each GEMM run on?  (one untimed pass)
     keyed = []
     for name, m, x in layers:
@@ -465,10 +553,15 @@ def main():
     n_dom = len(groups[dominant])
     total_ops = sum(o for *_, o in order)
 
+    by_name_b = {name: (m, x) for name, m, x in layers_b}
+    order_b = [(name, *by_name_b[name], ops) for name, _, _, ops in order]
+    flip = {"i": 0}
+
     def step(ev=None):
+        flip["i"] ^= 1
         if ev is not None:
             ev[0].record()
-        for i, (_, m, x, _) in enumerate(order):
+        for i, (_, m, x, _) in enumerate(order if flip["i"] else order_b):
             m(x)
             if ev is not None and i == n_dom - 1:
                 ev[1].record()
@@ -516,6 +609,8 @@ def main():
             "workload": "OPT-6.7B W8A8 linear set, M=2048 tokens (4x512), hidden 4096: q/k/v/out W8A8B8O8 "
                         "4096x4096, fc1 4096->16384 GELU-quant int8, fc2 16384->4096 fp32 out",
             "gemms_per_step": len(order),
+            "operand_sets": "2 sets of weights and activations (2 x 264 MB) alternate between steps: operands come from HBM, "
+                            "not from the 256 MB Infinity Cache",
             "int8_ops_per_step": total_ops,
             "kernels": {k: [n for n, *_ in v] for k, v in groups.items()},
         },
@@ -527,6 +622,7 @@ def main():
             "unit": "TFLOP/s",
             "frac": achieved / INT8_PEAK_TOPS,
             "traffic": MEASURED_TRAFFIC_BYTES.get(dominant),
+            "traffic_source": MEASURED_TRAFFIC_SOURCE.get(dominant),
             "algorithmic_bytes": sum(x.numel() + m.weight.numel() + x.shape[0] * m.weight.shape[0]
                                      for _, m, x, _ in groups[dominant]) / n_dom,
             "launches_per_step": n_dom,
@@ -541,10 +637,14 @@ def main():
     result["roofline"]["frac_of_measured_issue_peak"] = achieved / peak_rand
     if not args.no_extra:
         result["extra"] = extras(torch, dev)
+        result["extra"]["attention_i8_fused_vs_chain_40x2048x2048"] = attention_mismatch(torch, dev)
+        result["extra"]["m_sweep_K10240_N6848"] = m_sweep(torch, dev, 6848, 10240, lib)
+        result["extra"]["m_sweep_K5120_N5120"] = m_sweep(torch, dev, 5120, 5120, lib)
         result["extra"]["opt13b_decoder_layer"] = decoder_layer_ms(torch, dev)
         result["extra"]["sustained_fc2_2048x4096x16384"] = sustained_clock(torch, dev)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(torch, layers)
+        result["cpu_baseline"]["row_kernels"] = cpu_baseline_rows(torch)
     print(json.dumps(result))
 
 
