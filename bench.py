@@ -27,7 +27,7 @@ METRIC = "int8 GEMM TOPS (% MFMA peak), LN/GELU GB/s, W8A8 OPT-13B layer ms"
 # the launches of one step), from rocprofv3 FETCH_SIZE and WRITE_SIZE passes scaled by the same
 # counters' readings for a 256 MiB device copy (x2.0 and x1.0); see profiles/.
 MEASURED_TRAFFIC_BYTES = {
-    "ws_256x128x128_w2x2_s1_p3_l4/int8": (2.0 * 52601 + 1.0 * 15384) * 1024,
+    "ws_256x128x128_w2x2_s1_p3_l4/int8": (2.0 * 52606 + 1.0 * 14816) * 1024,
 }
 # where that reading comes from: the summary file and what the kernel's tile order was when it was
 # taken (the figure is only as fresh as that file; bench.py does not re-measure it)
@@ -485,6 +485,9 @@ def main():
     ap.add_argument("--bmm-qk-only", action="store_true",
                     help="run 4 launches of the Q.K^T BMM to int8 (160 x 2048 x 2048 x 128) and exit: the program "
                          "profiled for the Q.K^T counter summary")
+    ap.add_argument("--rownorm-only", action="store_true",
+                    help="run 6 launches of LayerNormQ and 3 of dq + add + LayerNormQ on 8192 x 5120 and exit: the "
+                         "program profiled for the row-norm counter summary")
     ap.add_argument("--calib-copy-mb", type=int, default=0,
                     help="before the timed region, run 4 device-to-device copies of this many MiB: a kernel of "
                          "known traffic to scale rocprofv3's FETCH_SIZE / WRITE_SIZE readings with")
@@ -511,6 +514,19 @@ def main():
         al, be = torch.tensor(0.002, device=dev), torch.tensor(0.01, device=dev)
         for i in range(24):
             linear.linear_a8_w8_b8_o8(x, ws[i % 6], b8, al, be)
+        torch.cuda.synchronize()
+        return
+    if args.rownorm_only:
+        from triton_int_amd.kernels import fused
+
+        rows, cols = 8192, 5120
+        xs = [torch.randn(rows, cols, device=dev) for _ in range(2)]
+        gam, bet = torch.randn(cols, device=dev) * 2 + 20, torch.randn(cols, device=dev) * 2
+        acc = torch.randint(-2**20, 2**20 + 1, (rows, cols), dtype=torch.int32, device=dev)
+        for i in range(6):
+            fused.layer_norm_fwd_fused_single_pass_q(xs[i & 1], gam, bet, 1e-5)
+        for i in range(3):
+            fused.dq_add_layernorm_q(acc, 1e-5, xs[i & 1], gam, bet, 1e-5)
         torch.cuda.synchronize()
         return
     if args.bmm_qk_only:
