@@ -390,6 +390,46 @@ def test_decode_shapes_skinny_kernel(M, N, K):
     assert mx <= 1 and rate < 1e-3
 
 
+@pytest.mark.parametrize("M,N,K", [(16, 5120, 4096), (16, 4096, 2048 + 48), (5, 2052, 3072), (16, 1024, 1024 + 16)])
+def test_decode_kernel_wave_layouts_bit_exact(M, N, K):
+    """The M <= 16 kernel with 8 streaming waves x 3 ring stages, 6 x 4 (what the library picks for 6
+    or fewer units of 4 weight rows per workgroup) and 4 x 6, and with K split over 2 / 4 / 8 waves
+    (forced through bits 8..15 of the configuration argument: low nibble the split, high nibble the
+    waves): every layout must give the oracle's bits for int32, int8 and fp32 outputs."""
+    linear, _, _ = _kl()
+    L = _lib()
+    lib = L.lib()
+    names = [lib.ti_gemm_config_name(i).decode() for i in range(lib.ti_gemm_num_configs())]
+    c = names.index("rows4_m16")
+    g = rng(M + N + K)
+    a, w = rand_i8(g, M, K, lo=-128), rand_i8(g, N, K, lo=-128)
+    b32 = g.integers(-2**20, 2**20, size=N, dtype=np.int32)
+    b8 = rand_i8(g, N); bf = g.standard_normal(N).astype(np.float32)
+    ga, gw, gb32, gb8, gbf = gpu(a), gpu(w), gpu(b32), gpu(b8), gpu(bf)
+    alpha = np.float32(40.0 / (np.sqrt(K) * 127 * 127 / 3)); beta = np.float32(0.05)
+    want32 = O.linear_a8_w8_b32_o32(a, w, b32)
+    want8 = O.linear_a8_w8_b8_o8(a, w, b8, alpha, beta)
+    wantf = O.linear_a8_w8_bfp32_ofp32(a, w, bf, alpha, 1.0)
+    per = -(-((N + 3) // 4) // 256)  # units per workgroup
+    ran = 0
+    for forced in (0, 1, 2, 4, 8, 0x80, 0x60, 0x40):
+        fits = ((forced >> 4) in (0, 8) or per <= (forced >> 4)) and ((forced & 15) <= 1 or per <= (8 // (forced & 15)) * 4)
+        cfg = c | (forced << 8)
+        if not fits:
+            with pytest.raises(AssertionError):  # TI_E_COMBO
+                linear.linear_a8_w8_b32_o32(ga, gw, gb32, _config=cfg)
+            continue
+        assert np.array_equal(cpu(linear.linear_a8_w8_b32_o32(ga, gw, gb32, _config=cfg)), want32), hex(forced)
+        assert np.array_equal(cpu(linear.linear_a8_w8_b8_o8(ga, gw, gb8, alpha, beta, _config=cfg)), want8), hex(forced)
+        assert np.array_equal(cpu(linear.linear_a8_w8_bfp32_ofp32(ga, gw, gbf, alpha, 1.0, _config=cfg)), wantf), hex(forced)
+        ran += 1
+    assert ran >= 5
+    with pytest.raises(AssertionError):
+        linear.linear_a8_w8_b32_o32(ga, gw, gb32, _config=c | (3 << 8))
+    with pytest.raises(AssertionError):
+        linear.linear_a8_w8_b32_o32(ga, gw, gb32, _config=c | (0x50 << 8))
+
+
 @pytest.mark.parametrize("M,N,K", [(130, 272, 2064), (300, 400, 1040), (64, 400, 4096), (33, 112, 2048), (700, 144, 4112)])
 def test_split_k_every_ws_config_bit_exact(M, N, K):
     """K dealt to 2..8 work items per tile (forced through bits 8..15 of the configuration argument):

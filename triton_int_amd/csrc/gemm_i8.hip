@@ -1531,6 +1531,9 @@ __global__ __launch_bounds__(512, UU ? 2 : 4) void gemm_skinny_kernel(GemmParams
 // LDS row pitches: activation rows are read 16 rows x 4 chunks at a time (pitch = 4 banks mod 64: the
 // 16 rows of a quarter wave hit 64 different banks); a weight job's 4 rows are read 4 rows x 4 chunks
 // with every address shared by 4 lanes (pitch = 16 banks mod 64: 16 different bank groups).
+// A workgroup with fewer units than waves lets only NWA of its 8 consumer waves stream, each with a
+// deeper ring (NWA x NST = 24 stages of 4 x 1 KB either way): what a wave can pull is bounded by the
+// bytes it keeps in flight, so 5 units on 5 waves x 3 stages leave a third of the CU's share unused.
 constexpr int R4_NW = 8, R4_RG = 4, R4_KC = 1024, R4_PITCH = R4_KC + 16, R4_WPITCH = R4_KC + 64, R4_NST = 3, R4_XB = 3,
               R4_UMAX = 4;
 
@@ -1544,7 +1547,7 @@ __device__ __attribute__((noinline)) void rows4_store_tile(const EpiCtx e, char*
                                                           int max_units, const float* resid, int64_t resid_rs, int bz,
                                                           const GemmParams* kp) {
   constexpr int ESZ = OUTCLS == OUT8 ? 1 : (OUTCLS == OUT32 ? 4 : 2);
-  constexpr int RING = R4_NST * R4_RG * R4_WPITCH;
+  constexpr int RING = R4_NST * R4_RG * R4_WPITCH;  // the tile's geometry, whatever the kernel's ring depth
   const int row = tid >> 5, grp = tid & 31;
   const int unit = unit0 + grp;
   if (!(row < M && unit < u_end && grp < max_units)) return;
@@ -1595,8 +1598,9 @@ __device__ __attribute__((noinline)) void rows4_store_tile(const EpiCtx e, char*
   }
 }
 
-template <int OUTCLS>
+template <int OUTCLS, int NWA, int NST>
 __global__ __launch_bounds__((R4_NW + 1) * 64) void gemm_rows4_kernel(GemmParams p) {
+  static_assert(NWA * NST == R4_NW * R4_NST && NWA <= R4_NW, "the rings share one LDS area");
   constexpr int STAGE = R4_RG * R4_WPITCH;  // one job: 4 rows x 1 KB (+ padding against bank conflicts)
   constexpr int XBUF = 16 * R4_PITCH;
   __shared__ __attribute__((aligned(16))) char lds[R4_XB * XBUF + R4_NW * R4_NST * STAGE];
@@ -1607,10 +1611,12 @@ __global__ __launch_bounds__((R4_NW + 1) * 64) void gemm_rows4_kernel(GemmParams
   const int OOB = (int)0x80000000;
   const int lda = (int)p.sAm, ldb = (int)p.sBn;
   const int NCH = (p.K + R4_KC - 1) / R4_KC;  // chunks of K
-  // KS = 2 (few weight rows): two waves share a unit and take the even / the odd chunks of K, so
-  // that all 8 waves stream; their partial sums meet in LDS at the end.  Only with a single pass.
-  const int KS = p.ksplit;
-  const int NSLOT = R4_NW / KS;  // units a workgroup works on at a time
+  // KS = 2, 4 or 8 (only when the host asks for it): KS waves share a unit and take the chunks
+  // kpart, kpart + KS, ... of K; their partial sums meet in LDS at the end.  Only with a single
+  // pass.  The waves of a unit then take turns at the chunk barriers, which is why the host prefers
+  // fewer streaming waves with deeper rings (NWA < 8) when a workgroup has few units.
+  const int KS = NWA == R4_NW ? p.ksplit : 1;
+  const int NSLOT = NWA / KS;  // units a workgroup works on at a time
   // units (groups of 4 weight rows) of this workgroup: [ub0, ub1), dealt to the slots round-robin,
   // at most NSLOT * R4_UMAX of them per pass over K
   const int NU = (p.N + R4_RG - 1) / R4_RG;
@@ -1649,10 +1655,12 @@ __global__ __launch_bounds__((R4_NW + 1) * 64) void gemm_rows4_kernel(GemmParams
   }
 
   // ---- consumers
-  const int slot = wave % NSLOT, kpart = wave / NSLOT;
+  // waves NWA..7 (kpart >= KS): no units, barriers only
+  const int slot = NWA == R4_NW ? wave % NSLOT : wave, kpart = NWA == R4_NW ? wave / NSLOT : (wave >= NWA ? 1 : 0);
   const v4i rW = make_rsrc(p.B + (int64_t)bz * p.sBb, (p.N - 1) * ldb + p.K);
-  const unsigned ring = lds_base + R4_XB * XBUF + wave * (R4_NST * STAGE);
-  char* ring_p = lds + R4_XB * XBUF + wave * (R4_NST * STAGE);
+  const int ring_i = wave < NWA ? wave : 0;
+  const unsigned ring = lds_base + R4_XB * XBUF + ring_i * (NST * STAGE);
+  char* ring_p = lds + R4_XB * XBUF + ring_i * (NST * STAGE);
   const int r16 = lane & 15, c4 = lane >> 4;
   const int w_lane = (r16 & (R4_RG - 1)) * R4_WPITCH + c4 * 16;  // rows 4..15 of the operand repeat rows 0..3
   const int x_lane = r16 * R4_PITCH + c4 * 16;
@@ -1665,18 +1673,18 @@ __global__ __launch_bounds__((R4_NW + 1) * 64) void gemm_rows4_kernel(GemmParams
   for (int pass = 0; pass < npass; ++pass) {
     const int u_first = ub0 + pass * (NSLOT * R4_UMAX) + slot;  // this wave's units: u_first + NSLOT*i, i < nu
     const int u_end = min(ub1, ub0 + (pass + 1) * (NSLOT * R4_UMAX));
-    const int nu = u_first < u_end ? (u_end - u_first + NSLOT - 1) / NSLOT : 0;
+    const int nu = (u_first < u_end && wave < NWA) ? (u_end - u_first + NSLOT - 1) / NSLOT : 0;
     const int njobs = nu * nch_mine;
-    // job j = (this wave's chunk number j / nu, unit j % nu): 4 loads of 1 KB, into ring slot j % 3;
+    // job j = (this wave's chunk number j / nu, unit j % nu): 4 loads of 1 KB, into ring slot j % NST;
     // beyond the last job the loads are redirected out of range (zeros into a slot nobody reads)
     // so that the number in flight stays constant
     auto issue_job = [&](int j) {
       const bool real = j < njobs;
       const int cm = real ? j / nu : 0, ui = real ? j - cm * nu : 0;
-      const int k0 = (kpart + cm * KS) * R4_KC;
+      const int k0 = __builtin_amdgcn_readfirstlane((kpart + cm * KS) * R4_KC);  // uniform; says so to the compiler
       const int row0 = (u_first + ui * NSLOT) * R4_RG;
       const bool in = real && k0 + kl < p.K;
-      const unsigned dst = ring + (j % R4_NST) * STAGE;
+      const unsigned dst = ring + (j % NST) * STAGE;
 #pragma unroll
       for (int r = 0; r < R4_RG; ++r)
         dma16_to_lds_stream(rW, in ? min(row0 + r, p.N - 1) * ldb + kl : OOB, k0, dst + r * R4_WPITCH);
@@ -1685,8 +1693,8 @@ __global__ __launch_bounds__((R4_NW + 1) * 64) void gemm_rows4_kernel(GemmParams
 #pragma unroll
     for (int i = 0; i < R4_UMAX; ++i) acc[i] = (v4i){0, 0, 0, 0};
     if (nu > 0) {
-      issue_job(0);
-      issue_job(1);
+#pragma unroll
+      for (int i = 0; i < NST - 1; ++i) issue_job(i);
     }
     int j = 0;
     for (int c = 0; c < NCH; ++c, ++g) {
@@ -1701,31 +1709,34 @@ __global__ __launch_bounds__((R4_NW + 1) * 64) void gemm_rows4_kernel(GemmParams
 #pragma unroll
       for (int ui = 0; ui < R4_UMAX; ++ui) {
         if (ui < nu) {
-          issue_job(j + 2);
-          asm volatile("s_waitcnt vmcnt(%0)" ::"n"(R4_RG * (R4_NST - 1)) : "memory");  // job j has landed
-          const char* wb = ring_p + (j % R4_NST) * STAGE + w_lane;
+          issue_job(j + NST - 1);
+          asm volatile("s_waitcnt vmcnt(%0)" ::"n"(R4_RG * (NST - 1)) : "memory");  // job j has landed
+          const char* wb = ring_p + (j % NST) * STAGE + w_lane;
 #pragma unroll
           for (int s = 0; s < 16; ++s)
             acc[ui] = __builtin_amdgcn_mfma_i32_16x16x64_i8(*(const v4i*)(wb + s * 64), xf[s], acc[ui], 0, 0, 0);
-          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // slot j % 3 is free for job j + 3
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // slot j % NST is free for job j + NST
           ++j;
         }
       }
     }
     if (nu > 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // trailing redirected loads
     if (KS > 1) {
-      // odd-chunk waves park their sums in their own (now idle) ring; the even-chunk partner adds them
-      if (kpart == 1) {
+      // the waves of the later chunks park their sums in their own (now idle) rings; the wave of the
+      // first chunks adds them
+      if (kpart > 0) {
 #pragma unroll
         for (int ui = 0; ui < R4_UMAX; ++ui)
           if (ui < nu) *(v4i*)(ring_p + ui * 1024 + lane * 16) = acc[ui];
       }
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
       if (kpart == 0) {
-        const char* other = ring_p + NSLOT * (R4_NST * STAGE);
+        for (int kp = 1; kp < KS; ++kp) {
+          const char* other = ring_p + kp * NSLOT * (NST * STAGE);
 #pragma unroll
-        for (int ui = 0; ui < R4_UMAX; ++ui)
-          if (ui < nu) acc[ui] += *(const v4i*)(other + ui * 1024 + lane * 16);
+          for (int ui = 0; ui < R4_UMAX; ++ui)
+            if (ui < nu) acc[ui] += *(const v4i*)(other + ui * 1024 + lane * 16);
+        }
       }
     }
     // ---- epilogue.  acc[ui][i], lanes 0..15: n = unit*4 + i, m = lane.  The workgroup's units of a pass
@@ -1821,7 +1832,7 @@ static const Config g_configs[] = {
     TI_WS(256, 128, 128, 2, 2, 1, 3, 4),
     TI_STREAM(128, 128, 64, 2, 2, 2, 3, 2),
     {"skinny_m16_slab32", {gemm_skinny_kernel<OUT8, 1, 2>, gemm_skinny_kernel<OUT32, 1, 2>, gemm_skinny_kernel<OUT16, 1, 2>}, 16, 32, 64, 512, true, true},
-    {"rows4_m16", {gemm_rows4_kernel<OUT8>, gemm_rows4_kernel<OUT32>, gemm_rows4_kernel<OUT16>}, 16, 4, 1024, (R4_NW + 1) * 64, true, false, 0, true},
+    {"rows4_m16", {gemm_rows4_kernel<OUT8, 8, 3>, gemm_rows4_kernel<OUT32, 8, 3>, gemm_rows4_kernel<OUT16, 8, 3>}, 16, 4, 1024, (R4_NW + 1) * 64, true, false, 0, true},
     TI_WS(256, 160, 128, 4, 1, 1, 3, 4),
     TI_WS(128, 128, 128, 2, 2, 1, 4, 4),
 };
@@ -1953,6 +1964,16 @@ static int pick_config(const GemmParams& p, int* splits_out) {
     if (best_cost < 0 || cost < best_cost) best_cost = cost, best = c.cfg, *splits_out = splits;
   }
   return best;
+}
+
+// gemm_rows4_kernel with nwa of its 8 consumer waves streaming (24 / nwa ring stages each)
+static KernelFn rows4_kernel(int oc, int nwa) {
+  static const KernelFn fns[3][3] = {
+      {gemm_rows4_kernel<OUT8, 8, 3>, gemm_rows4_kernel<OUT32, 8, 3>, gemm_rows4_kernel<OUT16, 8, 3>},
+      {gemm_rows4_kernel<OUT8, 6, 4>, gemm_rows4_kernel<OUT32, 6, 4>, gemm_rows4_kernel<OUT16, 6, 4>},
+      {gemm_rows4_kernel<OUT8, 4, 6>, gemm_rows4_kernel<OUT32, 4, 6>, gemm_rows4_kernel<OUT16, 4, 6>},
+  };
+  return fns[nwa == 6 ? 1 : (nwa == 4 ? 2 : 0)][oc];
 }
 
 static int pick_group_m(const GemmParams& p, const Config& k) {
@@ -2123,9 +2144,22 @@ static int run(GemmParams p, int config, hipStream_t stream, bool static_scratch
   if (k.stream_occ && !stream_eligible(p)) return fail(TI_E_COMBO, "config %s needs a row-major output with 16-byte aligned rows", k.name);
   if (k.rows4) {
     if (p.M > k.bm) return fail(TI_E_COMBO, "config %s needs M <= %d", k.name, k.bm);
-    // few weight rows: two waves per unit (even / odd chunks of K), so that every wave streams
+    // K is not split over waves unless a test asks for it: the waves of a unit take turns at the
+    // chunk barriers instead of streaming side by side (measured slower on every decode shape)
     const int units = (p.N + R4_RG - 1) / R4_RG;
-    p.ksplit = (units <= 1024 && p.K > R4_KC) ? 2 : 1;
+    p.ksplit = 1;
+    // forced by a test: low nibble the K split (1, 2, 4, 8), high nibble the streaming waves (4, 6, 8)
+    int want_nwa = 0;
+    if (want_splits) {
+      const int ks = want_splits & 15;
+      want_nwa = want_splits >> 4;
+      if (ks != 0 && ks != 1 && ks != 2 && ks != 4 && ks != 8)
+        return fail(TI_E_COMBO, "config %s splits K over 1, 2, 4 or 8 waves, not %d", k.name, ks);
+      if (want_nwa != 0 && want_nwa != 4 && want_nwa != 6 && want_nwa != 8)
+        return fail(TI_E_COMBO, "config %s streams on 4, 6 or 8 waves, not %d", k.name, want_nwa);
+      if (ks) p.ksplit = ks;
+      if (want_nwa && want_nwa != 8) p.ksplit = 1;
+    }
     // One workgroup per CU (its LDS allows no second one), all batches together in one round of
     // the 256 CUs, every CU busy: what a CU can pull from memory is the limit (about 27 GB/s each),
     // so an idle CU costs more than waves of a workgroup that carry one unit less than others
@@ -2133,8 +2167,19 @@ static int run(GemmParams p, int config, hipStream_t stream, bool static_scratch
     const int wgs = p.batch >= 256 ? 1 : 256 / p.batch;
     const int per = (units + wgs - 1) / wgs;
     const int blocks = (units + per - 1) / per;
+    // the K split needs all of a workgroup's units in one pass
+    if (p.ksplit > 1 && per > (R4_NW / p.ksplit) * R4_UMAX) {
+      if (want_splits) return fail(TI_E_COMBO, "config %s: %d units per workgroup do not fit one pass with K split over %d waves", k.name, per, p.ksplit);
+      p.ksplit = 1;
+    }
+    // 6 or fewer units per workgroup: 6 streaming waves with 4 ring stages each instead of 8 with 3
+    // (weights rotated through > 600 MB: 5120 x 20480 28.6 -> 25.3 us, 4096 x 16384 24.0 -> 20.0 us,
+    // 4096 x 4096 10.0 -> 8.7 us; 4 waves with 6 stages: equal or slower than 6 with 4)
+    int nwa = want_nwa ? want_nwa : (p.ksplit == 1 && per <= 6 ? 6 : 8);
+    if (nwa < 8 && per > nwa) return fail(TI_E_COMBO, "config %s: %d units per workgroup need more than %d waves", k.name, per, nwa);
     g_last_config = config;
-    k.fn[out_class(p.out_dtype)]<<<dim3((unsigned)blocks, (unsigned)p.batch), dim3(k.threads), 0, stream>>>(p);
+    g_last_splits = p.ksplit;
+    rows4_kernel(out_class(p.out_dtype), nwa)<<<dim3((unsigned)blocks, (unsigned)p.batch), dim3(k.threads), 0, stream>>>(p);
     return launch_status(k.name);
   }
   if (k.skinny) {
