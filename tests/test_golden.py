@@ -58,17 +58,21 @@ def test_gpu_gemm_fixture_all_epilogues_and_configs():
             continue  # that configuration takes fewer activation rows than the fixture has
         assert np.array_equal(_host(linear.linear_a8_w8_b32_o32(a, w, _dev(d["b32"]), _config=cfg)), d["o32"])
         assert np.array_equal(_host(linear.linear_a8_w8_b32_o32_with_scaling(a, w, _dev(d["b32"]), 0.01, be, _config=cfg)), d["o32_scaled"])
-        for name, rm in (("rne", 0), ("trunc", 1)):
+        for mode, rm in (("rne", 0), ("trunc", 1)):
             if rm == 1 and cfg > 0 and not name.startswith(("skinny", "rows4")):
                 continue  # truncation (test-time switch) is not implemented by the large-tile kernels
-            assert np.array_equal(_host(linear.linear_a8_w8_b8_o8(a, w, _dev(d["b8"]), al, be, _round_mode=rm, _config=cfg)), d[f"o8_{name}"])
-            assert np.array_equal(_host(linear.linear_relu_a8_w8_b8_o8(a, w, _dev(d["b8"]), al, be, _round_mode=rm, _config=cfg)), d[f"o8_relu_{name}"])
+            if name.startswith("shortk"):
+                continue  # the short-K kernel has no int8 epilogue with a bias or GELU
+            assert np.array_equal(_host(linear.linear_a8_w8_b8_o8(a, w, _dev(d["b8"]), al, be, _round_mode=rm, _config=cfg)), d[f"o8_{mode}"])
+            assert np.array_equal(_host(linear.linear_relu_a8_w8_b8_o8(a, w, _dev(d["b8"]), al, be, _round_mode=rm, _config=cfg)), d[f"o8_relu_{mode}"])
             got = _host(fused.linear_a8_w8_bfp32_ofp32_GeLu_Q(a, w, _dev(d["bf"]), float(d["ag"]), float(d["bg"]), _round_mode=rm, _config=cfg))
-            diff = np.abs(got.astype(int) - d[f"gelu_{name}"].astype(int))
+            diff = np.abs(got.astype(int) - d[f"gelu_{mode}"].astype(int))
             assert diff.max() <= 1 and (diff != 0).mean() < 1e-3
         assert np.array_equal(_host(linear.linear_a8_w8_bfp32_ofp32(a, w, _dev(d["bf"]), 0.0037, 1.0, _config=cfg)), d["of32"])
         assert np.array_equal(_host(linear.linear_a8_w8_bfp32_ofp32(a, w, _dev(d["bf"]), 0.0037, 1.0, dtype=torch.float16, _config=cfg)), d["of16"])
         assert np.array_equal(_host(linear.linear_a8_w8_bfp32_ofp32(a, w, _dev(d["bf"]), 0.0037, 1.0, dtype=torch.bfloat16, _config=cfg)), d["obf16"])
+        if name.startswith("shortk"):
+            continue  # K of the large fixture is beyond that kernel's 128
         assert np.array_equal(_host(linear.linear_a8_w8_b32_o32(_dev(d["big_a"]), _dev(d["big_w"]), None, _config=cfg)), d["big_o32"])
         assert np.array_equal(_host(linear.linear_a8_w8_ofp32(_dev(d["big_a"]), _dev(d["big_w"]), 1.0, _config=cfg)), d["big_of32"])
 

@@ -16,17 +16,20 @@ def _lib():
     return L
 
 
-def _configs(M=1, N=None, out8=False):
+def _configs(M=1, N=None, out8=False, K=None, bias8=True):
     """(index, name) of every kernel configuration that can run M activation rows (and, for the
-    persistent "stream" kernels with an int8 output, N output columns: they store whole 16-byte
-    segments of a row)"""
+    persistent kernels with an int8 output, N output columns: they store whole 16-byte segments of a
+    row; for the short-K kernel "shortk_..._k<max>", a K of 16..max and, for int8 outputs, neither bias
+    nor GELU: bias8=False says the int8 launches have none)"""
     L = _lib()
     n = L.lib().ti_gemm_num_configs()
     out = [(i, L.lib().ti_gemm_config_name(i).decode()) for i in range(n)]
     def fits(nm):  # "skinny_m<rows>_..." configurations take at most <rows> activation rows
         if nm.startswith(("skinny", "rows4")):
             return M <= int(nm.split("_")[1][1:])
-        if nm.startswith(("stream", "ws_")) and out8:
+        if nm.startswith("shortk_") and (not (K is not None and 16 <= K <= int(nm.rsplit("_k", 1)[1])) or (out8 and bias8)):
+            return False
+        if nm.startswith(("stream", "ws_", "shortk_")) and out8:
             return N is not None and N % 16 == 0
         return True
     return [(i, nm) for i, nm in out if fits(nm)]
@@ -50,7 +53,7 @@ def test_all_configs_int32_bit_exact(shape):
     bias = g.integers(-2**24, 2**24, size=N, dtype=np.int32)
     want = O.linear_a8_w8_b32_o32(a, w, bias)
     ga, gw, gb = gpu(a), gpu(w), gpu(bias)
-    for cfg, name in _configs(M):
+    for cfg, name in _configs(M, K=K):
         got = cpu(linear.linear_a8_w8_b32_o32(ga, gw, gb, _config=cfg))
         assert np.array_equal(got, want), f"config {name}"
     got = cpu(linear.linear_a8_w8_b32_o32(ga, gw, gb))
@@ -69,7 +72,7 @@ def test_all_configs_int8_epilogues_bit_exact(shape):
         want = O.linear_a8_w8_b8_o8(a, w, bias, alpha, beta)
         want_relu = O.linear_relu_a8_w8_b8_o8(a, w, bias, alpha, beta)
         want_tr = O.linear_a8_w8_b8_o8(a, w, bias, alpha, beta, round_mode=O.TRUNC)
-        for cfg, name in _configs(M, N, out8=True):
+        for cfg, name in _configs(M, N, out8=True, K=K):
             got = cpu(linear.linear_a8_w8_b8_o8(ga, gw, gb, alpha, beta, _config=cfg))
             assert np.array_equal(got, want), f"o8 config {name} alpha {alpha}"
             got = cpu(linear.linear_relu_a8_w8_b8_o8(ga, gw, gb, alpha, beta, _config=cfg))
@@ -98,7 +101,7 @@ def test_grouped_linear_equals_separate_linears(shape):
                            for i in range(G)], axis=1)
     ga, gw, gb, gal, gbe = gpu(a), gpu(w), gpu(bias), gpu(alphas), gpu(betas)
     ran = set()
-    for cfg, name in [(-1, "auto")] + _configs(M, N, out8=True):
+    for cfg, name in [(-1, "auto")] + _configs(M, N, out8=True, K=K):
         got = cpu(linear.linear_group_a8_w8_b8_o8(ga, gw, gb, gal, gbe, G, _config=cfg))
         assert got.shape == (M, G * N) and np.array_equal(got, want), f"config {name}"
         ran.add(name.split("_")[0])
@@ -123,7 +126,7 @@ def test_all_configs_float_and_scaled_i32(shape):
     want_b = O.linear_a8_w8_bfp32_ofp32(a, w, bias_f, alpha, beta, out_dtype=O.DT_BF16)
     want_nb = O.linear_a8_w8_ofp32(a, w, alpha)
     want_s = O.linear_a8_w8_b32_o32_with_scaling(a, w, bias_i, alpha, beta)
-    for cfg, name in _configs(M):
+    for cfg, name in _configs(M, K=K):
         got = cpu(linear.linear_a8_w8_bfp32_ofp32(ga, gw, gpu(bias_f), alpha, beta, _config=cfg))
         assert got.dtype == np.float32 and np.array_equal(got, want_f), f"f32 {name}"
         got = cpu(linear.linear_a8_w8_bfp32_ofp32(ga, gw, gpu(bias_f), alpha, beta, dtype=torch.float16, _config=cfg))
@@ -148,7 +151,7 @@ def test_all_configs_gelu_q(shape):
     want = O.linear_a8_w8_bfp32_ofp32_GeLu_Q(a, w, bias, alpha, beta)
     assert np.unique(want).size > 100  # the case really exercises the rounding, not only the clamp
     ga, gw, gb = gpu(a), gpu(w), gpu(bias)
-    for cfg, name in _configs(M, N, out8=True):
+    for cfg, name in _configs(M, N, out8=True, K=K):
         got = cpu(fused.linear_a8_w8_bfp32_ofp32_GeLu_Q(ga, gw, gb, alpha, beta, _config=cfg))
         mx, rate = mismatch_report(got, want)
         assert mx <= 1 and rate < 1e-3, f"{name}: max {mx} rate {rate}"
@@ -225,8 +228,8 @@ def test_bmm_fast_path_all_configs(B, M, N, K):
     alpha = np.float32(1e-3)
     want8 = O.bmm_s8t_s8n_s8t(a, b, alpha)
     wantf = O.bmm_s8t_s8n_f32t(a, b, alpha)
-    out8_ok = {c for c, _ in _configs(M, N, out8=True)}
-    for cfg, name in _configs(M):
+    out8_ok = {c for c, _ in _configs(M, N, out8=True, K=K, bias8=False)}
+    for cfg, name in _configs(M, K=K):
         assert np.array_equal(cpu(bmm.bmm_s8t_s8n_s32t(ga, gb, _config=cfg)), want32), name
         if cfg in out8_ok:
             assert np.array_equal(cpu(bmm.bmm_s8t_s8n_s8t(ga, gb, alpha, _config=cfg)), want8), name
@@ -248,8 +251,8 @@ def test_stream_configs_many_tiles_per_workgroup(B, M, N, K):
     want8 = O.bmm_s8t_s8n_s8t(a, b, alpha)
     wantf = O.bmm_s8t_s8n_f32t(a, b, alpha)
     ran = 0
-    for cfg, name in _configs(M, N, out8=True):
-        if not name.startswith(("stream", "ws_")):
+    for cfg, name in _configs(M, N, out8=True, K=K, bias8=False):
+        if not name.startswith(("stream", "ws_", "shortk_")):
             continue
         ran += 1
         assert np.array_equal(cpu(bmm.bmm_s8t_s8n_s32t(ga, gb, _config=cfg)), want32), name

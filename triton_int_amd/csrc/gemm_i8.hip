@@ -609,7 +609,9 @@ constexpr int epi_strip_bytes(int wtn) { return ((wtn / 16) & (wtn / 16 - 1)) ==
 #ifndef TI_STREAM_STORE32_AUX
 #define TI_STREAM_STORE32_AUX 2
 #endif
-template <int TM, int TN, int OUTCLS>
+// LDS_COLS false: `strip` has no room for the column terms; int8 launches with a bias or GELU are not
+// compiled in (the host refuses them for such a kernel).
+template <int TM, int TN, int OUTCLS, bool LDS_COLS = true>
 __device__ __forceinline__ void stream_epilogue(const GemmParams& p, const EpiCtx& e, v16i (&acc)[TM][TN], int bz,
                                                 int mw, int nw, char* strip, int lane) {
   constexpr int WTN = TN * 32;
@@ -699,10 +701,14 @@ __device__ __forceinline__ void stream_epilogue(const GemmParams& p, const EpiCt
       }
     };
     const bool gelu = e.epilogue == TI_EPI_GELU_I8;
-    if (gelu && has_bias) body(std::true_type{}, std::true_type{});
-    else if (gelu) body(std::true_type{}, std::false_type{});
-    else if (has_bias) body(std::false_type{}, std::true_type{});
-    else body(std::false_type{}, std::false_type{});
+    if constexpr (!LDS_COLS) {
+      body(std::false_type{}, std::false_type{});
+    } else {
+      if (gelu && has_bias) body(std::true_type{}, std::true_type{});
+      else if (gelu) body(std::true_type{}, std::false_type{});
+      else if (has_bias) body(std::false_type{}, std::true_type{});
+      else body(std::false_type{}, std::false_type{});
+    }
   } else {
     // acc[i][j][r]: m = mw + i*32 + 8*(r/4) + 4*lhi + r%4;  n = nw + j*32 + lrow.
     // KIND: 0 raw int32 (+ int32 bias), 1 scaled -> int32, 2 scaled -> fp32, 3 -> fp16, 4 -> bf16
@@ -985,6 +991,160 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
   }
   // the trailing (empty-buffer) loads still write zeros into LDS: they must land before the
   // workgroup's LDS is handed to another one
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+// ---- short-K persistent kernel -------------------------------------------------------------------
+//
+// K <= 128 (the attention Q.K^T: K is the head dimension): a 256 x 256 tile is 32 MFMAs per wave
+// against 128 outputs per lane to scale, clamp, round, pack and store; the k-loop machinery of
+// gemm_mfma_stream_kernel (a barrier and a wait per k-tile, loads dealt over the k-steps) buys nothing
+// here.  The whole K of a tile sits in LDS (two tile buffers: one being read, one being loaded) and
+// there is one barrier per tile: every wave issues its share of tile t+1's loads right after
+// barrier t (into the buffer of tile t-1: all of its readers passed that barrier), runs tile t's
+// MFMAs and epilogue, and waits for those loads before barrier t+1; the only younger operations are
+// the epilogue's unconditional stores, so the count to wait for is exact.
+// 4 x 2 waves of 64 x 128 outputs: an int8 row piece of a wave is a whole 128-byte line (with 2 x 4
+// waves it is 64 bytes, and a write-only probe of this output pattern runs at 3.5 TB/s with 64-byte
+// pieces against 5.3-5.6 TB/s with 128 bytes and more).  The 32 x 128-byte strips of the 8 waves
+// and the two tile buffers fill the 160 KB of LDS exactly: there is no room to stage per-column
+// terms, so int8 launches with a bias or the GELU epilogue go to the other kernels (the BMMs have
+// neither).
+// Tried and removed: a ping-pong order (the two waves of a SIMD in opposite order between barriers,
+// one wave's MFMAs under the other's epilogue), 9-16 % slower than this order for every pairing of
+// waves (160 x 2048 x 2048 x 128: 193 us against 209-224 us).
+template <int OUTCLS>
+__global__ __launch_bounds__(512) void gemm_mfma_shortk_kernel(GemmParams p) {
+  constexpr int BM = 256, BN = 256, BK = 64, WAVES_N = 2, SWZ = 2, KTMAX = 2;
+  constexpr int NT = 512, CH = BK / 16;
+  constexpr int WTM = 64, WTN = 128, TM = WTM / 32, TN = WTN / 32;
+  constexpr int A_BYTES = BM * BK, B_BYTES = BN * BK, STAGE = A_BYTES + B_BYTES, TILE = KTMAX * STAGE;
+  constexpr int STRIP = epi_strip_bytes(WTN);
+  constexpr int EPI_LDS = OUTCLS == OUT8 ? 8 * STRIP : 0;
+  constexpr int LDS_BYTES = 2 * TILE + EPI_LDS;
+  constexpr int STORES_ALL = OUTCLS == OUT8 ? TM * TN : TM * TN * 16;  // store instructions per tile and wave
+  constexpr int STORES = STORES_ALL > 63 ? 63 : STORES_ALL;            // 63: the counter's maximum (waits longer)
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+
+  __shared__ __attribute__((aligned(16))) char lds[LDS_BYTES];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+  // ---- this workgroup's items (as in gemm_mfma_stream_kernel)
+  const int T = p.tiles_m * p.tiles_n;
+  const int W = T * p.batch;
+  int first, step, count;
+  {
+    const int G = (int)gridDim.x, b = (int)blockIdx.x;
+    if (G & 7) {
+      first = b;
+      step = G;
+      count = b < W ? (W - b + G - 1) / G : 0;
+    } else {
+      const int xcd = b & 7, l = b >> 3, nb = G >> 3;
+      const int per = W >> 3, rem = W & 7;
+      const int cnt = per + (xcd < rem ? 1 : 0);
+      first = xcd * per + min(xcd, rem) + l;
+      step = nb;
+      count = l < cnt ? (cnt - l + nb - 1) / nb : 0;
+    }
+    first = __builtin_amdgcn_readfirstlane(first);
+    step = __builtin_amdgcn_readfirstlane(step);
+    count = __builtin_amdgcn_readfirstlane(count);
+  }
+  if (count == 0) return;
+  auto locate = [&](int i, int& bz, int& m0, int& n0) {
+    const int g = first + i * step;
+    const int b_ = g / T;
+    int tm, tn;
+    tile_from_rank(p, g - b_ * T, tm, tn);
+    bz = __builtin_amdgcn_readfirstlane(b_);
+    m0 = __builtin_amdgcn_readfirstlane(tm * BM);
+    n0 = __builtin_amdgcn_readfirstlane(tn * BN);
+  };
+
+  const int lda = (int)p.sAm, ldb = (int)p.sBn;
+  const unsigned lds_base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+  const unsigned wave_slot = __builtin_amdgcn_readfirstlane(lds_base + wave * 1024);
+  TileLoader<BM, BK, NT, SWZ> la;
+  TileLoader<BN, BK, NT, SWZ> lb;
+  la.init(tid, 0, lda, p.K);
+  lb.init(tid, 0, ldb, p.K);
+  constexpr int A_IT = decltype(la)::IT, B_IT = decltype(lb)::IT;
+  const int KT = (p.K + BK - 1) / BK;  // 1 or 2 (host)
+  const int OOB = (int)0x80000000;
+
+  // all of item i's K into tile buffer buf; rows at or past M (N) and bytes past K read as zero
+  auto load_tile = [&](int i, int buf) {
+    int bz, m0, n0;
+    locate(i, bz, m0, n0);
+    const v4i rA = make_rsrc(p.A + (int64_t)bz * p.sAb + (int64_t)m0 * lda, (p.M - 1 - m0) * lda + p.K);
+    const v4i rB = make_rsrc(p.B + (int64_t)bz * p.sBb + (int64_t)n0 * ldb, (p.N - 1 - n0) * ldb + p.K);
+#pragma unroll
+    for (int kt = 0; kt < KTMAX; ++kt) {
+      if (kt < KT) {
+        const int k0 = kt * BK;
+        const unsigned dst = wave_slot + buf * TILE + kt * STAGE;
+#pragma unroll
+        for (int d = 0; d < A_IT; ++d) dma16_to_lds(rA, (k0 < la.klim[d]) ? la.voff[d] : OOB, k0, dst + d * NT * 16);
+#pragma unroll
+        for (int d = 0; d < B_IT; ++d) dma16_to_lds(rB, (k0 < lb.klim[d]) ? lb.voff[d] : OOB, k0, dst + A_BYTES + d * NT * 16);
+      }
+    }
+  };
+
+  v16i acc[TM][TN];
+  const int frow = lane & 31;
+  const int fsw = (frow >> SWZ) & (CH - 1);
+  const int fhalf = lane >> 5;
+  const int a_lane = (wm * WTM + frow) * BK;
+  const int b_lane = A_BYTES + (wn * WTN + frow) * BK;
+  v4i fa[2][TM], fb[2][TN];
+  constexpr int NM = TM * TN, NR = TM + TN;
+  auto load_frag = [&](const char* stage, int ks, int buf, int r) {
+    const int coff = ((ks * 2 + fhalf) ^ fsw) * 16;
+    if (r < TM) fa[buf][r] = *(const v4i*)(stage + a_lane + r * 32 * BK + coff);
+    else fb[buf][r - TM] = *(const v4i*)(stage + b_lane + (r - TM) * 32 * BK + coff);
+  };
+  // one k-step: the MFMAs on fragment set buf, the reads of the next k-step's fragments (set buf ^ 1)
+  // spread between them; first: the sums start from a zero C operand
+  auto kstep = [&](int buf, const char* rd_stage, int rd_ks, bool do_read, auto first_tag) {
+    const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int u = 0; u < NM; ++u) {
+      const int i = u / TN, j = u % TN;
+      const v16i c = decltype(first_tag)::value ? zero : acc[i][j];
+      if constexpr (OUTCLS == OUT8) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[buf][j], fa[buf][i], c, 0, 0, 0);
+      else acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[buf][i], fb[buf][j], c, 0, 0, 0);
+      if (do_read && u < NR) load_frag(rd_stage, rd_ks, buf ^ 1, u);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+
+  load_tile(0, 0);
+  for (int t = 0; t < count; ++t) {
+    // this wave's loads of tile t have landed and its LDS reads are done; then meet the others.  The
+    // operations younger than those loads are the stores of tile t-1's epilogue.
+    if (t >= 1) wait_loads_and_barrier<STORES>();
+    else wait_loads_and_barrier<0>();
+    if (t + 1 < count) load_tile(t + 1, (t + 1) & 1);
+    const char* s0 = lds + (t & 1) * TILE;
+#pragma unroll
+    for (int r = 0; r < NR; ++r) load_frag(s0, 0, 0, r);
+    kstep(0, s0, 1, true, std::true_type{});
+    if (KT == 2) {
+      kstep(1, s0 + STAGE, 0, true, std::false_type{});
+      kstep(0, s0 + STAGE, 1, true, std::false_type{});
+    }
+    kstep(1, s0, 0, false, std::false_type{});
+    int bz, m0, n0;
+    locate(t, bz, m0, n0);
+    const EpiCtx e = make_epi(p, bz);
+    stream_epilogue<TM, TN, OUTCLS, false>(p, e, acc, bz, m0 + wm * WTM, n0 + wn * WTN, lds + 2 * TILE + wave * STRIP, lane);
+  }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
@@ -1772,6 +1932,7 @@ struct Config {
   int stream_occ = 0;   // > 0: gemm_mfma_stream_kernel, this many workgroups per CU walk the tile list
   bool rows4 = false;   // gemm_rows4_kernel: M <= 16
   int ws_waves = 0;     // > 0: gemm_mfma_ws_kernel with this many consumer waves (it can split K)
+  int max_k = 0;        // > 0: the kernel holds a tile's whole K in LDS and takes 16 <= K <= max_k only
 };
 
 #define TI_FAST(BM, BN, BK, WM, WN, SWZ, NS)                                              \
@@ -1817,6 +1978,7 @@ enum ConfigId {
   CFG_ROWS4_16,      // M <= 16, K >= 1024: weights streamed as 1 KB row pieces
   CFG_WS_256x160,    // 2048 x 5120 outputs are exactly 256 of these tiles: one full round of the chip
   CFG_WS_128x128,    // few activation rows and a long K: split K over enough of these to fill the chip
+  CFG_SHORTK_256x256,  // K <= 128 (attention Q.K^T): a tile's whole K in LDS, one barrier per tile, 128-byte int8 row pieces
 };
 
 static const Config g_configs[] = {
@@ -1835,6 +1997,8 @@ static const Config g_configs[] = {
     {"rows4_m16", {gemm_rows4_kernel<OUT8, 8, 3>, gemm_rows4_kernel<OUT32, 8, 3>, gemm_rows4_kernel<OUT16, 8, 3>}, 16, 4, 1024, (R4_NW + 1) * 64, true, false, 0, true},
     TI_WS(256, 160, 128, 4, 1, 1, 3, 4),
     TI_WS(128, 128, 128, 2, 2, 1, 4, 4),
+    {"shortk_256x256x64_w4x2_k128", {gemm_mfma_shortk_kernel<OUT8>, gemm_mfma_shortk_kernel<OUT32>, gemm_mfma_shortk_kernel<OUT16>}, 256, 256, 64, 512,
+     true, false, 1, false, 0, 128},
 };
 static const int g_num_configs = (int)(sizeof(g_configs) / sizeof(g_configs[0]));
 
@@ -1944,6 +2108,11 @@ static int pick_config(const GemmParams& p, int* splits_out) {
     return CFG_WS_128x128;
   }
   if (p.M <= 64) return CFG_SKINNY_16 + (p.M > 16) + (p.M > 32);
+  // K <= 128, int8 out, at least two 256 x 256 tiles per workgroup: the epilogue is most of the work
+  if (stream && p.K >= 16 && p.K <= g_configs[CFG_SHORTK_256x256].max_k && out_class(p.out_dtype) == OUT8 &&
+      (!p.bias || p.bias_kind == TI_BIAS_NONE) && p.epilogue != TI_EPI_GELU_I8 &&
+      (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch >= 512)
+    return CFG_SHORTK_256x256;
   // short K: the epilogue dominates and the larger tile halves the operand traffic per output
   const double big = p.K <= 512 ? 1.20 : 0.97;
   struct Cand { int cfg; double eff; };
@@ -2142,6 +2311,9 @@ static int run(GemmParams p, int config, hipStream_t stream, bool static_scratch
   if (k.fast && !k.skinny && !k.rows4 && trunc8) return fail(TI_E_COMBO, "config %s does not implement TI_ROUND_TRUNC for int8 outputs", k.name);
   if (k.fast && !fast_eligible(p)) return fail(TI_E_COMBO, "config %s needs K-contiguous 16-byte aligned operands", k.name);
   if (k.stream_occ && !stream_eligible(p)) return fail(TI_E_COMBO, "config %s needs a row-major output with 16-byte aligned rows", k.name);
+  if (k.max_k && (p.K < 16 || p.K > k.max_k)) return fail(TI_E_COMBO, "config %s needs 16 <= K <= %d", k.name, k.max_k);
+  if (k.max_k && out_class(p.out_dtype) == OUT8 && (p.bias_kind != TI_BIAS_NONE || p.epilogue == TI_EPI_GELU_I8))
+    return fail(TI_E_COMBO, "config %s has no int8 epilogue with a bias or GELU", k.name);
   if (k.rows4) {
     if (p.M > k.bm) return fail(TI_E_COMBO, "config %s needs M <= %d", k.name, k.bm);
     // K is not split over waves unless a test asks for it: the waves of a unit take turns at the
