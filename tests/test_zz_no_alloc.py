@@ -35,7 +35,7 @@ def test_static_scratch_entry_point_matches_the_allocating_one():
     # left in the scratch must not leak into the second
     for (M, N, K, cfg_name, splits) in [(200, 1040, 8192, "ws_128x128", 7), (96, 272, 2064, "ws_128x128", 3),
                                         (300, 528, 4112, "ws_256x128", 4), (130, 400, 1040, "ws_256x160", 2),
-                                        (128, 6848, 10240, None, 0), (64, 1024, 4096, None, 0)]:
+                                        (128, 6848, 10240, None, 0), (64, 1024, 8192, None, 0)]:
         g = rng(M + N + K)
         a, w = rand_i8(g, M, K, lo=-128), rand_i8(g, N, K, lo=-128)
         b8, bf = rand_i8(g, N), g.standard_normal(N).astype(np.float32)
@@ -81,7 +81,7 @@ def test_static_scratch_rejects_what_does_not_fit_and_is_capturable():
     assert _call(lib.ti_bmm_i8_static_scratch, ga, gw, gbf, alpha, beta, out, L.EPI_SCALE_F, -1) == 0
     assert torch.equal(out, want)
     # captured on a stream that never had a workspace: replays give the eager result every time
-    M, N, K = 128, 1024, 4096
+    M, N, K = 128, 1024, 8192
     ga, gw, gbf = gpu(rand_i8(g, M, K)), gpu(rand_i8(g, N, K)), gpu(g.standard_normal(N).astype(np.float32))
     out = torch.empty((M, N), dtype=torch.float32, device=DEV)
     want = torch.empty_like(out)

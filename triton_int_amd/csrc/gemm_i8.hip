@@ -2069,14 +2069,14 @@ static double config_cost(const GemmParams& p, const Config& k, double eff, int 
 }
 
 // Number of K splits for a wave-specialised configuration: as many as fill the chip's 256 workgroup
-// slots once, but no split shorter than 2048 bytes of K and no more than 8 (the last item of a tile
-// reads the other splits' sums one after the other).
+// slots once, but no split shorter than 2560 bytes of K (K = 4096 is faster whole, K = 5120 in two
+// parts) and no more than 8 (the last item of a tile reads the other splits' sums one after the other).
 static int pick_splits(const GemmParams& p, const Config& k, double eff, double* cost_out) {
   int want = 1;
   if (k.ws_waves && p.batch == 1) {
     const int64_t tiles = (int64_t)((p.M + k.bm - 1) / k.bm) * ((p.N + k.bn - 1) / k.bn);
     const int64_t fill = tiles > 0 ? 256 / tiles : 1;
-    const int by_k = p.K / 2048;
+    const int by_k = p.K / 2560;
     want = (int)(fill < by_k ? fill : by_k);
     want = want < 1 ? 1 : (want > 8 ? 8 : want);
   }
@@ -2120,7 +2120,7 @@ static int pick_config(const GemmParams& p, int* splits_out) {
       {stream ? CFG_STREAM_256x256 : CFG_TILE_256x256, stream ? big : 1.00},
       {stream ? CFG_WS_256x128 : CFG_TILE_256x128, stream ? 1.00 : 0.90},
       {stream ? CFG_STREAM_128x128 : CFG_TILE_128x128, 0.78},
-      {CFG_TILE_64x64, 0.25},
+      {CFG_TILE_64x64, 0.20},
       {stream ? CFG_WS_256x160 : -1, 1.00},
       {stream ? CFG_WS_128x128 : -1, 0.85},
   };
@@ -2409,8 +2409,11 @@ static int run(GemmParams p, int config, hipStream_t stream, bool static_scratch
   if (k.stream_occ) {
     const int64_t items = (int64_t)p.tiles_m * p.tiles_n * p.batch * p.splits;
     if (items > 0x7fffffff) return fail(TI_E_SHAPE, "too many tiles");
+    // a multiple of 8 keeps workgroup b on XCD b % 8; rounded up, so that no workgroup gets a second
+    // item while CUs are idle (162 items on 160 workgroups took twice the time of 162 on 168; the
+    // workgroups without an item return at once)
     int64_t g = items < 256 * k.stream_occ ? items : 256 * k.stream_occ;
-    if (g >= 8) g &= ~(int64_t)7;  // a multiple of 8 keeps workgroup b on XCD b % 8
+    if (g >= 8) g = (g + 7) & ~(int64_t)7;
     k.fn[out_class(p.out_dtype)]<<<dim3((unsigned)g), dim3(k.threads), 0, stream>>>(p);
     return launch_status(k.name);
   }
