@@ -264,6 +264,12 @@ def extras(torch, dev):
     sc = torch.empty((B, S, S), dtype=torch.int8, device=dev)
     ms = time_region(torch, lambda: bmm.bmm_s8t_s8n_s8t(q, k, 1e-3, out=sc), 10, 2)
     out["bmm_qk_s8_160x2048x2048x128"] = {"ms": ms, "GBps": 755.0e6 / ms / 1e6, "TOPS": 171.8e9 / ms / 1e9}
+    # the same launch on all-zero operands: same instructions and bytes, less switching in the MFMAs
+    # and data paths, so the chip holds a higher clock (what the kernel does when power is not the limit)
+    qz, kz = torch.zeros_like(q), torch.zeros_like(k)
+    ms = time_region(torch, lambda: bmm.bmm_s8t_s8n_s8t(qz, kz, 1e-3, out=sc), 10, 2)
+    out["bmm_qk_s8_160x2048x2048x128_zero_operands"] = {"ms": ms, "GBps": 755.0e6 / ms / 1e6, "TOPS": 171.8e9 / ms / 1e9}
+    del qz, kz
     # probabilities as the baseline prescribes them: round(127 * softmax(N(0,1) * s)), here from this
     # library's own softmax-quantise kernel on int8 scores round(32 * N(0,1)) with scale 0.05 (logit std 1.6)
     p = fused.softmax_q(torch.randn((B, S, S), device=dev).mul_(32).round_().clamp_(-127, 127).to(torch.int8), 0.05)
@@ -311,6 +317,25 @@ def extras(torch, dev):
     out["single_linear_512x768x768"] = {"eager_us": eager_ms * 1e3, "graph_us": graph_ms * 1e3,
                                         "TOPS_graph": 2.0 * 512 * 768 * 768 / (graph_ms * 1e-3) / 1e12}
     del x1, w1, b1, o1
+    # q/k/v of the linear set as three launches on one input and as one grouped launch (what the decoder
+    # layer does): 768 tiles in one launch instead of three single-round launches
+    xq = torch.randint(-127, 128, (2048, 4096), dtype=torch.int8, device=dev)
+    w3 = torch.randint(-127, 128, (3 * 4096, 4096), dtype=torch.int8, device=dev)
+    b3 = torch.randint(-127, 128, (3 * 4096,), dtype=torch.int8, device=dev)
+    al3, be3 = torch.rand(3, device=dev) * 9e-3 + 1e-3, torch.rand(3, device=dev) * 9e-3 + 1e-3
+    o3 = torch.empty((2048, 3 * 4096), dtype=torch.int8, device=dev)
+    outs = [torch.empty((2048, 4096), dtype=torch.int8, device=dev) for _ in range(3)]
+
+    def three():
+        for i in range(3):
+            linear.linear_a8_w8_b8_o8(xq, w3[i * 4096:(i + 1) * 4096], b3[i * 4096:(i + 1) * 4096], al3[i], be3[i], out=outs[i])
+
+    t3 = time_region(torch, three, 20, 3)
+    tg = time_region(torch, lambda: linear.linear_group_a8_w8_b8_o8(xq, w3, b3, al3, be3, 3, out=o3), 20, 3)
+    ops3 = 3 * 2.0 * 2048 * 4096 * 4096
+    out["qkv_2048x3x4096x4096"] = {"three_launches_ms": t3, "three_launches_TOPS": ops3 / t3 / 1e9,
+                                   "grouped_launch_ms": tg, "grouped_launch_TOPS": ops3 / tg / 1e9}
+    del xq, w3, b3, o3, outs
     # a yardstick, not part of the path: the vendor library's int8 GEMM (torch._int_mm, int32 out) on
     # the fc1 shape with the same kind of operands, next to this library's int32-output linear
     try:
