@@ -233,7 +233,12 @@ static int launch_layernorm_fp(const LnFpParams& p, hipStream_t stream) {
     return launch_status("layernorm_fp_any_kernel");
   }
   const int vpt = (p.cols / N + LF_THREADS - 1) / LF_THREADS;
-  const unsigned slots = 256u * (vpt <= 2 ? 8u : (vpt <= 5 ? 4u : 2u));
+  // persistent workgroups per CU for 3..5 vectors per thread, measured at 16384 rows of 5120 / 4096
+  // columns with 4 / 3 / 2 of them: the skip variants (two or three streams per row) run best with 2
+  // (fp16 122 / 114 / 113 us, bf16 122 / 117 / 110, fp32 244 / 246 / 232), plain fp32 with 3 at 5120
+  // columns (118 / 113 / 113) and 2 at 4096 (94 / 93 / 88), plain 16-bit with 4 (56 / 60 / 80)
+  const unsigned mid = p.skip ? 2u : (sizeof(T) == 4 ? (vpt >= 5 ? 3u : 2u) : 4u);
+  const unsigned slots = 256u * (vpt <= 2 ? 8u : (vpt <= 5 ? mid : 2u));
   const dim3 grid((unsigned)p.rows < slots ? (unsigned)p.rows : slots), block(LF_THREADS);
 #define TI_LF_LAUNCH(V) layernorm_fp_vec_kernel<T, V><<<grid, block, 0, stream>>>(p)
   if (vpt <= 1) TI_LF_LAUNCH(1);
