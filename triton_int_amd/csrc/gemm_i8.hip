@@ -2109,10 +2109,12 @@ static int pick_config(const GemmParams& p, int* splits_out) {
   }
   if (p.M <= 64) return CFG_SKINNY_16 + (p.M > 16) + (p.M > 32);
   // K <= 128, int8 out, at least two 256 x 256 tiles per workgroup: the epilogue is most of the work
+  // (and tiles that are mostly output, not padding)
   if (stream && p.K >= 16 && p.K <= g_configs[CFG_SHORTK_256x256].max_k && out_class(p.out_dtype) == OUT8 &&
-      (!p.bias || p.bias_kind == TI_BIAS_NONE) && p.epilogue != TI_EPI_GELU_I8 &&
-      (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch >= 512)
-    return CFG_SHORTK_256x256;
+      (!p.bias || p.bias_kind == TI_BIAS_NONE) && p.epilogue != TI_EPI_GELU_I8) {
+    const int64_t tm = (p.M + 255) / 256, tn = (p.N + 255) / 256;
+    if (tm * tn * p.batch >= 512 && (double)p.M * p.N >= 0.6 * (double)(tm * 256) * (double)(tn * 256)) return CFG_SHORTK_256x256;
+  }
   // short K: the epilogue dominates and the larger tile halves the operand traffic per output
   const double big = p.K <= 512 ? 1.20 : 0.97;
   struct Cand { int cfg; double eff; };
