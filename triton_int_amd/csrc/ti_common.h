@@ -51,17 +51,19 @@ __device__ __forceinline__ unsigned pack4(int a, int b, int c, int d) {
 }
 
 // tanh-GELU times scale, 0.5 * x * (1 + tanh(k * (x + 0.044715 * x^3))) * scale
-// (kernels/fused.py:79), evaluated as x * (1 - 1 / (1 + e^(2u))) * scale with
-// 2u * log2(e) = (2 k log2 e) * x * (1 + 0.044715 x^2): 8 plain operations, one exp2 and one
-// reciprocal per element instead of 15 + 2 in the literal order — in a GEMM epilogue this is
-// time the matrix pipe waits.  Same function to within a few fp32 ulps; after the int8
-// quantisation a value sitting on a rounding boundary can come out one step apart.
+// (kernels/fused.py:79), evaluated as (x * scale) / (1 + e^(-2u)) with
+// -2u * log2(e) = x * (c0 + c1 * x^2), c0 = -2 k log2 e, c1 = 0.044715 * c0: 6 plain operations, one
+// exp2 and one reciprocal per element instead of 15 + 2 in the literal order — in a GEMM epilogue
+// this is time the matrix pipe waits.  Same function to within a few fp32 ulps (no cancellation at
+// either end: e -> inf gives x * scale * 0, e -> 0 gives x * scale); after the int8 quantisation a
+// value sitting on a rounding boundary can come out one step apart.
 __device__ __forceinline__ float gelu_tanh_scaled(float x, float scale) {
-  const float c1 = 2.30220819814f;  // 2 * sqrt(2/pi) * log2(e)
-  const float p = __builtin_fmaf(x * x, 0.044715f, 1.0f);
-  const float e = __builtin_amdgcn_exp2f((x * p) * c1);
+  const float c0 = -2.30220819814f;            // -2 * sqrt(2/pi) * log2(e)
+  const float c1 = -2.30220819814f * 0.044715f;
+  const float p = __builtin_fmaf(x * x, c1, c0);
+  const float e = __builtin_amdgcn_exp2f(x * p);
   const float r = __builtin_amdgcn_rcpf(1.0f + e);
-  return (x * (1.0f - r)) * scale;
+  return (x * scale) * r;
 }
 
 // ---- softmax-quantise arithmetic -----------------------------------------------------------------
