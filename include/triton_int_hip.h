@@ -123,8 +123,12 @@ int ti_bmm_i8(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk,
  * to 0xff = choose the configuration): K is dealt to that many work items per tile, whose int32
  * partial sums meet in a workspace the library keeps per device and stream (allocated on first
  * use, up to 96 MiB; never during a graph capture, where an unsplit launch is used if there is
- * none yet).  Integer sums: the result does not depend on the split.  Returns TI_E_COMBO if the
- * configuration cannot run the given stride pattern or cannot split K.
+ * none yet).  Integer sums: the result does not depend on the split.  For the M <= 16
+ * weight-streaming configuration ("rows4_m16") the same bits select its wave layout instead: low
+ * nibble the number of waves that share a unit of weight rows along K (1, 2, 4, 8), high nibble
+ * the number of streaming waves (4, 6, 8); 0 = choose.  Returns TI_E_COMBO if the configuration
+ * cannot run the given shape or stride pattern (e.g. "shortk_..." takes 16 <= K <= 128 and, for
+ * int8 outputs, neither bias nor GELU) or cannot split K that way.
  */
 int ti_bmm_i8_config(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk,
                      const int8_t* B, int64_t sBb, int64_t sBn, int64_t sBk,
