@@ -2122,7 +2122,7 @@ static int pick_config(const GemmParams& p, int* splits_out) {
       {stream ? CFG_STREAM_256x256 : CFG_TILE_256x256, stream ? big : 1.00},
       {stream ? CFG_WS_256x128 : CFG_TILE_256x128, stream ? 1.00 : 0.90},
       {stream ? CFG_STREAM_128x128 : CFG_TILE_128x128, 0.78},
-      {CFG_TILE_64x64, 0.20},
+      {CFG_TILE_64x64, 0.25},
       {stream ? CFG_WS_256x160 : -1, 1.00},
       {stream ? CFG_WS_128x128 : -1, 0.85},
   };
