@@ -139,6 +139,32 @@ def test_all_configs_float_and_scaled_i32(shape):
         assert np.array_equal(got, want_s), f"scaled i32 {name}"
 
 
+def test_half_outputs_paired_and_single_stores():
+    """fp16 / bf16 outputs go out as dword pairs where a row keeps pairs aligned (even N, even pitch,
+    4-byte aligned base) and element by element otherwise: both ways give the oracle's bits, and the
+    columns around a view stay untouched."""
+    linear, _, _ = _kl()
+    g = rng(77)
+    alpha, beta = np.float32(0.0037), np.float32(0.71)
+    for (M, N, K, pitch, col0) in ((300, 272, 384, 272, 0),    # pairs
+                                  (300, 273, 384, 273, 0),    # odd N: single elements
+                                  (300, 272, 384, 281, 0),    # odd pitch
+                                  (300, 272, 384, 280, 3),    # view starting at an odd element
+                                  (300, 272, 384, 280, 4),    # view at an even element: pairs inside a wider matrix
+                                  (513, 130, 128, 130, 0)):
+        a, w = rand_i8(g, M, K), rand_i8(g, N, K)
+        bias_f = g.standard_normal(N).astype(np.float32)
+        ga, gw, gb = gpu(a), gpu(w), gpu(bias_f)
+        for dt, odt in ((torch.float16, O.DT_F16), (torch.bfloat16, O.DT_BF16)):
+            want = O.linear_a8_w8_bfp32_ofp32(a, w, bias_f, alpha, beta, out_dtype=odt)
+            for cfg, name in [(-1, "auto")] + _configs(M, K=K):
+                wide = torch.zeros((M, pitch), dtype=dt, device=DEV)
+                linear.linear_a8_w8_bfp32_ofp32(ga, gw, gb, alpha, beta, dtype=dt, out=wide[:, col0:col0 + N], _config=cfg)
+                got = wide.view(torch.int16).cpu().numpy().view(np.uint16)
+                assert np.array_equal(got[:, col0:col0 + N], want.view(np.uint16)), f"{(M, N, K, pitch, col0)} {dt} {name}"
+                assert not got[:, :col0].any() and not got[:, col0 + N:].any(), f"outside the view: {(M, N, K, pitch, col0)} {name}"
+
+
 @pytest.mark.parametrize("shape", SHAPES[:3], ids=lambda s: "x".join(map(str, s)))
 def test_all_configs_gelu_q(shape):
     _, _, fused = _kl()

@@ -609,6 +609,10 @@ constexpr int epi_strip_bytes(int wtn) { return ((wtn / 16) & (wtn / 16 - 1)) ==
 #ifndef TI_STREAM_STORE32_AUX
 #define TI_STREAM_STORE32_AUX 2
 #endif
+// 2-byte outputs: pairs of neighbouring elements of a row can go out as one aligned dword
+__device__ __forceinline__ bool out16_pairs(const GemmParams& p) {
+  return !(p.N & 1) && !(p.sCm & 1) && !(p.sCb & 1) && !((uintptr_t)p.C & 3);
+}
 // LDS_COLS false: `strip` has no room for the column terms; int8 launches with a bias or GELU are not
 // compiled in (the host refuses them for such a kernel).
 template <int TM, int TN, int OUTCLS, bool LDS_COLS = true>
@@ -712,32 +716,116 @@ __device__ __forceinline__ void stream_epilogue(const GemmParams& p, const EpiCt
   } else {
     // acc[i][j][r]: m = mw + i*32 + 8*(r/4) + 4*lhi + r%4;  n = nw + j*32 + lrow.
     // KIND: 0 raw int32 (+ int32 bias), 1 scaled -> int32, 2 scaled -> fp32, 3 -> fp16, 4 -> bf16
+    // A store's address is split: the lane's part (its column and its first row, or the out-of-range
+    // offset) is one VGPR per column block, the row's part R * pitch rides in the instruction's scalar
+    // offset, which the range check ignores; a row beyond M swaps the lane part for the out-of-range
+    // offset.  Per store that is a compare and a select, no multiply and no branch.
+    const int pitch = ldc * ESZ;
+    const int rows_left = p.M - mw - 4 * lhi;
     auto body = [&](auto kind_tag) {
       constexpr int KIND = decltype(kind_tag)::value;
+      if constexpr (KIND == 3 || KIND == 4) {
+        // 2-byte outputs whose rows keep pairs of elements dword-aligned: straight from the MFMA layout a
+        // store instruction would write 64 separate 2-byte pieces.  Instead (a) the upper half-wave of
+        // column block j is exchanged with the lower half-wave of block j+1 (v_permlane32_swap), which
+        // leaves a register with one row's 64 consecutive elements, and (b) even and odd lanes trade
+        // elements of two such rows (one DPP move), so that even lanes hold dwords of row m and odd lanes
+        // dwords of row m+1: half the store instructions, each writing two whole 128-byte lines.
+        if (out16_pairs(p)) {
+          const int odd = lane & 1;
+          const int rows_left_pair = p.M - mw - odd;
+#pragma unroll
+          for (int j = 0; j + 1 < TN; j += 2) {
+            float col2[2];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) col2[h] = column_term_t<TI_BIAS_F32>(e, min(nw + (j + h) * 32 + lrow, p.N - 1), false);
+            const int n = nw + (j + lhi) * 32 + (lrow & ~1);  // first element of the lane's dword; N is even
+            const int base = n < p.N ? ((mw + odd) * ldc + n) * ESZ : OOB;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+#pragma unroll
+              for (int r = 0; r < 16; r += 2) {
+                unsigned row[2][2];  // [r, r+1][lower, upper half-wave's row]
+#pragma unroll
+                for (int rr = 0; rr < 2; ++rr) {
+                  unsigned bits[2];
+#pragma unroll
+                  for (int h = 0; h < 2; ++h) {
+                    float v = (float)acc[i][j + h][r + rr] * e.alpha;
+                    const float vb = col2[h] + v;
+                    v = has_bias ? vb : v;
+                    bits[h] = KIND == 3 ? (unsigned)f32_to_f16_bits(v) : (unsigned)f32_to_bf16_bits(v);
+                  }
+                  const auto sw = __builtin_amdgcn_permlane32_swap(bits[0], bits[1], false, false);
+                  row[rr][0] = sw[0];
+                  row[rr][1] = sw[1];
+                }
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                  const unsigned lo_row = row[0][h], hi_row = row[1][h];  // rows m and m + 1, element n of each
+                  const unsigned give = odd ? lo_row : hi_row;
+                  const unsigned got = (unsigned)__builtin_amdgcn_mov_dpp((int)give, 0xB1, 0xf, 0xf, true);  // lane ^ 1
+                  const unsigned dword = odd ? (got | (hi_row << 16)) : (lo_row | (got << 16));
+                  const int R = i * 32 + 8 * (r >> 2) + 4 * h + (r & 3);  // row mw + R + odd
+                  __builtin_amdgcn_raw_buffer_store_b32(dword, rC, R < rows_left_pair ? base : OOB, R * pitch, TI_STREAM_STORE32_AUX);
+                }
+              }
+            }
+          }
+          if constexpr (TN % 2 == 1) {
+            // the last column block has no partner: step (b) alone, 64-byte pieces of rows m and m + 1
+            constexpr int j = TN - 1;
+            const float col = column_term_t<TI_BIAS_F32>(e, min(nw + j * 32 + lrow, p.N - 1), false);
+            const int n = nw + j * 32 + (lrow & ~1);
+            const int base = n < p.N ? ((mw + 4 * lhi + odd) * ldc + n) * ESZ : OOB;
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+#pragma unroll
+              for (int r = 0; r < 16; r += 2) {
+                unsigned row[2];
+#pragma unroll
+                for (int rr = 0; rr < 2; ++rr) {
+                  float v = (float)acc[i][j][r + rr] * e.alpha;
+                  const float vb = col + v;
+                  v = has_bias ? vb : v;
+                  row[rr] = KIND == 3 ? (unsigned)f32_to_f16_bits(v) : (unsigned)f32_to_bf16_bits(v);
+                }
+                const unsigned give = odd ? row[0] : row[1];
+                const unsigned got = (unsigned)__builtin_amdgcn_mov_dpp((int)give, 0xB1, 0xf, 0xf, true);
+                const unsigned dword = odd ? (got | (row[1] << 16)) : (row[0] | (got << 16));
+                const int R = i * 32 + 8 * (r >> 2) + (r & 3);  // row mw + R + 4 * lhi + odd
+                __builtin_amdgcn_raw_buffer_store_b32(dword, rC, R < rows_left - odd ? base : OOB, R * pitch, TI_STREAM_STORE32_AUX);
+              }
+            }
+          }
+          return;
+        }
+      }
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         const int n = nw + j * 32 + lrow;
         const int nc = min(n, p.N - 1);
         const float col = KIND == 0 ? 0.0f : column_term_t<KIND == 1 ? TI_BIAS_I32 : TI_BIAS_F32>(e, nc, false);
         const int bias_i32 = (KIND == 0 && e.bias_kind == TI_BIAS_I32) ? ((const int*)e.bias)[nc] : 0;
-        const bool n_ok = n < p.N;
+        const int base = n < p.N ? ((mw + 4 * lhi) * ldc + n) * ESZ : OOB;
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const int m = mw + i * 32 + 8 * (r >> 2) + 4 * lhi + (r & 3);
-            const int off = (n_ok && m < p.M) ? (m * ldc + n) * ESZ : OOB;
+            const int R = i * 32 + 8 * (r >> 2) + (r & 3);  // row mw + R + 4 * lhi
+            const int off = R < rows_left ? base : OOB;
+            const int soff = R * pitch;
             const int a = acc[i][j][r];
             if constexpr (KIND == 0) {
-              __builtin_amdgcn_raw_buffer_store_b32((unsigned)a + (unsigned)bias_i32, rC, off, 0, TI_STREAM_STORE32_AUX);
+              __builtin_amdgcn_raw_buffer_store_b32((unsigned)a + (unsigned)bias_i32, rC, off, soff, TI_STREAM_STORE32_AUX);
             } else {
               float v = (float)a * e.alpha;
               const float vb = col + v;
               v = has_bias ? vb : v;
-              if constexpr (KIND == 1) __builtin_amdgcn_raw_buffer_store_b32((unsigned)q32(v, e.round_mode), rC, off, 0, TI_STREAM_STORE32_AUX);
-              else if constexpr (KIND == 2) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rC, off, 0, TI_STREAM_STORE32_AUX);
-              else if constexpr (KIND == 3) __builtin_amdgcn_raw_buffer_store_b16(f32_to_f16_bits(v), rC, off, 0, 0);
-              else __builtin_amdgcn_raw_buffer_store_b16(f32_to_bf16_bits(v), rC, off, 0, 0);
+              if constexpr (KIND == 1) __builtin_amdgcn_raw_buffer_store_b32((unsigned)q32(v, e.round_mode), rC, off, soff, TI_STREAM_STORE32_AUX);
+              else if constexpr (KIND == 2) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rC, off, soff, TI_STREAM_STORE32_AUX);
+              else if constexpr (KIND == 3) __builtin_amdgcn_raw_buffer_store_b16(f32_to_f16_bits(v), rC, off, soff, 0);
+              else __builtin_amdgcn_raw_buffer_store_b16(f32_to_bf16_bits(v), rC, off, soff, 0);
             }
           }
         }
@@ -938,6 +1026,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
   constexpr int LOADS_A = LOADS - LOADS_B;
   constexpr int N_STEADY = LOADS * (DEPTH - 2) + LOADS_A;
   constexpr int N_AFTER_STORES = (N_STEADY + STORES > 63) ? 63 : N_STEADY + STORES;
+  // 2-byte outputs stored as dword pairs take half the store instructions
+  constexpr bool CAN_PAIR = OUTCLS == OUT16;
+  constexpr int N_AFTER_PAIRED = (N_STEADY + STORES / 2 > 63) ? 63 : N_STEADY + STORES / 2;
+  const bool paired = CAN_PAIR && out16_pairs(p);
 
   // ---- fill the pipeline
   aim(0);
@@ -979,7 +1071,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
       // all LDS reads of this k-tile are issued; the next k-tile must have landed before the
       // barrier.  The stores of the previous item's epilogue are younger than that k-tile while
       // it is one of those that were fetched before the epilogue.
-      if (it > 0 && kt < DEPTH - 1) wait_loads_and_barrier<N_AFTER_STORES>();
+      if (it > 0 && kt < DEPTH - 1) {
+        if (paired) wait_loads_and_barrier<N_AFTER_PAIRED>();
+        else wait_loads_and_barrier<N_AFTER_STORES>();
+      }
       else wait_loads_and_barrier<N_STEADY>();
       kstep((KS - 1) & 1, lds + st * STAGE, 0, kt + 1 < KT, LOADS_A, LOADS_B, std::false_type{});
       dma_advance();
