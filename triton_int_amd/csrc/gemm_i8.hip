@@ -595,7 +595,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3
 // Stores one wave's (TM*32) x (TN*32) block of accumulators, whose first row / column in the
 // output are mw / nw, through an unconditional, range-checked buffer store per element group
 // (elements outside M x N are redirected out of the buffer's range and dropped), so that the
-// number of store instructions per tile is a compile-time constant.  `strip` is the wave's private
+// number of store instructions per tile does not depend on the tile (2-byte outputs: one of two
+// constants, by out16_pairs()).  `strip` is the wave's private
 // LDS area (int8 outputs only): 32*WTN bytes for the row strip plus WTN floats of column terms.
 #ifndef TI_STREAM_STORE_AUX
 #define TI_STREAM_STORE_AUX 2  // nt: the outputs are streamed, keep the operand panels in L2
@@ -863,9 +864,10 @@ __device__ __forceinline__ void stream_epilogue(const GemmParams& p, const EpiCt
 // range and dropped by the range check).  A count too small would only wait longer; 63 is the
 // counter's maximum.
 //
-// The epilogue touches no LDS: 4-byte and 2-byte outputs are stored straight from the MFMA layout
-// (32 consecutive n per row and instruction), int8 outputs exchange dwords between the two wave
-// halves so that every lane owns 16 consecutive bytes of a row.
+// 4-byte outputs are stored straight from the MFMA layout (32 consecutive n per row and
+// instruction), 2-byte outputs as dword pairs after a lane exchange where the output's alignment
+// allows, int8 outputs exchange dwords between the two wave halves so that every lane owns 16
+// consecutive bytes of a row and go through a wave-private LDS strip.
 template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int SWZ, int NSTAGE, int OUTCLS, int OCC = 1>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64, (WAVES_M * WAVES_N * OCC + 3) / 4) void gemm_mfma_stream_kernel(GemmParams p) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
