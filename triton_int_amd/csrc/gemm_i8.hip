@@ -647,6 +647,17 @@ __device__ __forceinline__ void stream_epilogue(const GemmParams& p, const EpiCt
     const float q_floor = e.epilogue == TI_EPI_SCALE_RELU_I8 ? 0.0f : -128.0f;
     const int w_swz = (lrow / WRAP) & (SEG - 1);
     const int r_row = lane / SEG, r_seg = lane % SEG;
+    // Store addresses: the lane's own part (its column and its first row, or the out-of-range offset:
+    // 2^31, which stays out of range with a row's offset added) is computed once, the part that changes
+    // from store to store is a scalar added to it.  Not in the instruction's scalar-offset field as for
+    // the 4-byte stores below: the compiler puts no wait state between a 16-byte buffer store with a
+    // register in that field and a following VALU write of the store's data registers, and this GPU
+    // needs one (the first data dword of some lanes came out overwritten).
+    // N % 16 == 0: a 16-byte segment is wholly inside or outside.
+    const int s_rows_left = p.M - mw - r_row;                                           // via the strip
+    const int s_base = nw + r_seg * 16 < p.N ? (mw + r_row) * ldc + nw + r_seg * 16 : OOB;
+    const int d_rows_left = p.M - mw - lrow, d_cols_left = p.N - nw - lhi * 16;         // direct
+    const int d_base = (mw + lrow) * ldc + nw + lhi * 16;
     auto body = [&](auto gelu_tag, auto bias_tag) {
       constexpr bool GELU = decltype(gelu_tag)::value;
       constexpr bool BIAS = decltype(bias_tag)::value;
@@ -686,10 +697,8 @@ __device__ __forceinline__ void stream_epilogue(const GemmParams& p, const EpiCt
           } else {
             // no strip for this tile width: the lane stores its 16 bytes of row lrow itself (an
             // instruction touches 32 rows with 32 bytes each; left to L2 to merge into lines)
-            const int m = mw + i * 32 + lrow;
-            const int n = nw + (2 * j + lhi) * 16;
-            const int off = (m < p.M && n < p.N) ? m * ldc + n : OOB;
-            __builtin_amdgcn_raw_buffer_store_b128(v, rC, off, 0, 0);
+            const bool in = i * 32 < d_rows_left && j * 32 < d_cols_left;
+            __builtin_amdgcn_raw_buffer_store_b128(v, rC, (in ? d_base : OOB) + (i * 32 * ldc + j * 32), 0, 0);
           }
         }
         if constexpr (VIA_STRIP) {
@@ -697,10 +706,8 @@ __device__ __forceinline__ void stream_epilogue(const GemmParams& p, const EpiCt
           for (int q = 0; q < TN; ++q) {
             const int row = q * RP + r_row;
             const v4u v = *(const v4u*)(strip + row * WTN + ((r_seg ^ ((row / WRAP) & (SEG - 1))) * 16));
-            const int m = mw + i * 32 + row;
-            const int n = nw + r_seg * 16;
-            const int off = (m < p.M && n < p.N) ? m * ldc + n : OOB;  // N % 16 == 0: a segment is in or out
-            __builtin_amdgcn_raw_buffer_store_b128(v, rC, off, 0, TI_STREAM_STORE_AUX);
+            const int R = i * 32 + q * RP;  // row mw + R + r_row
+            __builtin_amdgcn_raw_buffer_store_b128(v, rC, (R < s_rows_left ? s_base : OOB) + R * ldc, 0, TI_STREAM_STORE_AUX);
           }
         }
       }
@@ -735,25 +742,35 @@ __device__ __forceinline__ void stream_epilogue(const GemmParams& p, const EpiCt
         if (out16_pairs(p)) {
           const int odd = lane & 1;
           const int rows_left_pair = p.M - mw - odd;
+          // per pair of column blocks: the two column terms and the lane part of the address; the loops
+          // run rows outside, column blocks inside, so that a row's range test serves all its stores
+          constexpr int NP = TN / 2;
+          float col2[NP > 0 ? NP : 1][2];
+          int base2[NP > 0 ? NP : 1];
 #pragma unroll
-          for (int j = 0; j + 1 < TN; j += 2) {
-            float col2[2];
+          for (int jp = 0; jp < NP; ++jp) {
 #pragma unroll
-            for (int h = 0; h < 2; ++h) col2[h] = column_term_t<TI_BIAS_F32>(e, min(nw + (j + h) * 32 + lrow, p.N - 1), false);
-            const int n = nw + (j + lhi) * 32 + (lrow & ~1);  // first element of the lane's dword; N is even
-            const int base = n < p.N ? ((mw + odd) * ldc + n) * ESZ : OOB;
+            for (int h = 0; h < 2; ++h) col2[jp][h] = column_term_t<TI_BIAS_F32>(e, min(nw + (2 * jp + h) * 32 + lrow, p.N - 1), false);
+            const int n = nw + (2 * jp + lhi) * 32 + (lrow & ~1);  // first element of the lane's dword; N is even
+            base2[jp] = n < p.N ? ((mw + odd) * ldc + n) * ESZ : OOB;
+          }
 #pragma unroll
-            for (int i = 0; i < TM; ++i) {
+          for (int i = 0; i < TM; ++i) {
 #pragma unroll
-              for (int r = 0; r < 16; r += 2) {
+            for (int r = 0; r < 16; r += 2) {
+              bool in[2];
+#pragma unroll
+              for (int h = 0; h < 2; ++h) in[h] = i * 32 + 8 * (r >> 2) + 4 * h + (r & 3) < rows_left_pair;
+#pragma unroll
+              for (int jp = 0; jp < NP; ++jp) {
                 unsigned row[2][2];  // [r, r+1][lower, upper half-wave's row]
 #pragma unroll
                 for (int rr = 0; rr < 2; ++rr) {
                   unsigned bits[2];
 #pragma unroll
                   for (int h = 0; h < 2; ++h) {
-                    float v = (float)acc[i][j + h][r + rr] * e.alpha;
-                    const float vb = col2[h] + v;
+                    float v = (float)acc[i][2 * jp + h][r + rr] * e.alpha;
+                    const float vb = col2[jp][h] + v;
                     v = has_bias ? vb : v;
                     bits[h] = KIND == 3 ? (unsigned)f32_to_f16_bits(v) : (unsigned)f32_to_bf16_bits(v);
                   }
@@ -768,7 +785,7 @@ __device__ __forceinline__ void stream_epilogue(const GemmParams& p, const EpiCt
                   const unsigned got = (unsigned)__builtin_amdgcn_mov_dpp((int)give, 0xB1, 0xf, 0xf, true);  // lane ^ 1
                   const unsigned dword = odd ? (got | (hi_row << 16)) : (lo_row | (got << 16));
                   const int R = i * 32 + 8 * (r >> 2) + 4 * h + (r & 3);  // row mw + R + odd
-                  __builtin_amdgcn_raw_buffer_store_b32(dword, rC, R < rows_left_pair ? base : OOB, R * pitch, TI_STREAM_STORE32_AUX);
+                  __builtin_amdgcn_raw_buffer_store_b32(dword, rC, in[h] ? base2[jp] : OOB, R * pitch, TI_STREAM_STORE32_AUX);
                 }
               }
             }
@@ -802,26 +819,33 @@ __device__ __forceinline__ void stream_epilogue(const GemmParams& p, const EpiCt
           return;
         }
       }
+      // rows outside, column blocks inside: a row's range test serves all its stores
+      float col[TN];
+      int bias_i32[TN], base[TN];
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         const int n = nw + j * 32 + lrow;
         const int nc = min(n, p.N - 1);
-        const float col = KIND == 0 ? 0.0f : column_term_t<KIND == 1 ? TI_BIAS_I32 : TI_BIAS_F32>(e, nc, false);
-        const int bias_i32 = (KIND == 0 && e.bias_kind == TI_BIAS_I32) ? ((const int*)e.bias)[nc] : 0;
-        const int base = n < p.N ? ((mw + 4 * lhi) * ldc + n) * ESZ : OOB;
+        col[j] = KIND == 0 ? 0.0f : column_term_t<KIND == 1 ? TI_BIAS_I32 : TI_BIAS_F32>(e, nc, false);
+        bias_i32[j] = (KIND == 0 && e.bias_kind == TI_BIAS_I32) ? ((const int*)e.bias)[nc] : 0;
+        base[j] = n < p.N ? ((mw + 4 * lhi) * ldc + n) * ESZ : OOB;
+      }
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
+      for (int i = 0; i < TM; ++i) {
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int R = i * 32 + 8 * (r >> 2) + (r & 3);  // row mw + R + 4 * lhi
-            const int off = R < rows_left ? base : OOB;
-            const int soff = R * pitch;
+        for (int r = 0; r < 16; ++r) {
+          const int R = i * 32 + 8 * (r >> 2) + (r & 3);  // row mw + R + 4 * lhi
+          const bool in = R < rows_left;
+          const int soff = R * pitch;
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+            const int off = in ? base[j] : OOB;
             const int a = acc[i][j][r];
             if constexpr (KIND == 0) {
-              __builtin_amdgcn_raw_buffer_store_b32((unsigned)a + (unsigned)bias_i32, rC, off, soff, TI_STREAM_STORE32_AUX);
+              __builtin_amdgcn_raw_buffer_store_b32((unsigned)a + (unsigned)bias_i32[j], rC, off, soff, TI_STREAM_STORE32_AUX);
             } else {
               float v = (float)a * e.alpha;
-              const float vb = col + v;
+              const float vb = col[j] + v;
               v = has_bias ? vb : v;
               if constexpr (KIND == 1) __builtin_amdgcn_raw_buffer_store_b32((unsigned)q32(v, e.round_mode), rC, off, soff, TI_STREAM_STORE32_AUX);
               else if constexpr (KIND == 2) __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rC, off, soff, TI_STREAM_STORE32_AUX);
