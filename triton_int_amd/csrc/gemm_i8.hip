@@ -264,6 +264,9 @@ struct TileLoader {
 // it, which drains the load pipeline once per k-tile and defeats multi-stage prefetching.  With
 // the loads invisible to that tracking, the kernel counts them itself (vmcnt retires in order).
 // M0 carries the LDS destination of a wave's 64 x 16 bytes; nothing else in these kernels uses M0.
+// The descriptor and the scalar offset handed to these helpers must come from scalar instructions
+// (kernel arguments, SALU arithmetic): the wait states a VMEM read of a VALU-written SGPR needs are
+// the compiler's job, and it does not look inside the asm.
 __device__ __forceinline__ v4i make_rsrc(const void* base, int bytes) {
   const uint64_t a = (uint64_t)base;
   v4i r;
@@ -1962,7 +1965,11 @@ __global__ __launch_bounds__((R4_NW + 1) * 64) void gemm_rows4_kernel(GemmParams
     auto issue_job = [&](int j) {
       const bool real = j < njobs;
       const int cm = real ? j / nu : 0, ui = real ? j - cm * nu : 0;
-      const int k0 = __builtin_amdgcn_readfirstlane((kpart + cm * KS) * R4_KC);  // uniform; says so to the compiler
+      // uniform; says so to the compiler.  The copy makes the register the loads read one that a scalar
+      // instruction wrote: a VMEM instruction must not read an SGPR within 5 wait states of a VALU
+      // instruction (v_readfirstlane) writing it, and the compiler does not see the loads inside the asm.
+      int k0 = __builtin_amdgcn_readfirstlane((kpart + cm * KS) * R4_KC);
+      asm volatile("s_mov_b32 %0, %1" : "=s"(k0) : "s"(k0));
       const int row0 = (u_first + ui * NSLOT) * R4_RG;
       const bool in = real && k0 + kl < p.K;
       const unsigned dst = ring + (j % NST) * STAGE;
