@@ -2192,8 +2192,12 @@ static double config_cost(const GemmParams& p, const Config& k, double eff, int 
   if (want > 1 && k.ws_waves && p.batch == 1) sk_shape(kt, want, splits, kt_split);
   const int64_t items = tm * tn * p.batch * splits;
   const int64_t rounds = (items + slots - 1) / slots;
+  // a last round that fills only part of the chip runs faster than a full one (the busy CUs share the
+  // power and the memory system of the idle ones): 2.5 rounds of 256 x 128 tiles measure like 2.7-2.8
+  const double idle = 1.0 - (double)(items - (rounds - 1) * slots) / (double)slots;
+  const double rounds_eff = (double)rounds - (rounds > 1 ? 0.4 : 0.2) * idle;
   const double k_len = (double)kt_split * k.bk + 512.0 + (splits > 1 ? 512.0 + 768.0 * splits : 0.0);
-  return (double)rounds * k_len * (double)(k.bm * k.bn) * occ / eff / (1.0 + 0.1 / (double)rounds);
+  return rounds_eff * k_len * (double)(k.bm * k.bn) * occ / eff / (1.0 + 0.1 / (double)rounds);
 }
 
 // Number of K splits for a wave-specialised configuration: as many as fill the chip's 256 workgroup
@@ -2209,7 +2213,12 @@ static int pick_splits(const GemmParams& p, const Config& k, double eff, double*
     want = want < 1 ? 1 : (want > 8 ? 8 : want);
   }
   int used = 1;
-  const double cost = config_cost(p, k, eff, want, used);
+  double cost = config_cost(p, k, eff, want, used);
+  if (used > 1) {  // whole K may still be the cheaper of the two
+    int one = 1;
+    const double whole = config_cost(p, k, eff, 1, one);
+    if (whole <= cost) cost = whole, used = 1;
+  }
   if (cost_out) *cost_out = cost;
   return used;
 }
@@ -2244,15 +2253,21 @@ static int pick_config(const GemmParams& p, int* splits_out) {
     if (tm * tn * p.batch >= 512 && (double)p.M * p.N >= 0.6 * (double)(tm * 256) * (double)(tn * 256)) return CFG_SHORTK_256x256;
   }
   // short K: the epilogue dominates and the larger tile halves the operand traffic per output
-  const double big = p.K <= 512 ? 1.20 : 0.97;
+  const double big = p.K <= 512 ? 1.20 : 0.92;
+  // 256 x 160 tiles: as good as 256 x 128 per unit of work with 2- and 4-byte outputs; with int8 outputs
+  // the tile has no LDS room left for the epilogue's row strip and stores 32-byte pieces (measured per
+  // output column, 2048 x 5120 x 5120: 0.32 us against 0.27 us).  Still the choice where it saves a
+  // round: 2048 x 5120 outputs are one round of 256 such tiles (56 us against 74 us), 2048 x 20480 take
+  // four rounds of them or five of the narrower tile (199 us against 182 us)
+  const double wide160 = out_class(p.out_dtype) == OUT8 ? 0.80 : 1.00;
   struct Cand { int cfg; double eff; };
   const Cand cands[] = {
       {stream ? CFG_STREAM_256x256 : CFG_TILE_256x256, stream ? big : 1.00},
       {stream ? CFG_WS_256x128 : CFG_TILE_256x128, stream ? 1.00 : 0.90},
-      {stream ? CFG_STREAM_128x128 : CFG_TILE_128x128, 0.78},
+      {stream ? CFG_STREAM_128x128 : CFG_TILE_128x128, stream ? 0.70 : 0.78},
       {CFG_TILE_64x64, 0.25},
-      {stream ? CFG_WS_256x160 : -1, 1.00},
-      {stream ? CFG_WS_128x128 : -1, 0.85},
+      {stream ? CFG_WS_256x160 : -1, wide160},
+      {stream ? CFG_WS_128x128 : -1, 0.80},
   };
   int best = CFG_TILE_64x64;
   double best_cost = -1.0;
