@@ -186,6 +186,28 @@ const char* ti_gemm_config_name(int config);
 int ti_gemm_last_config(void);
 /* Number of K splits that launch used (1 = K not split). */
 int ti_gemm_last_splits(void);
+/*
+ * Dry run of ti_bmm_i8_config (static_scratch != 0: of ti_bmm_i8_static_scratch): takes every decision
+ * the launch would take, through the same host code (validation, choice of configuration, K split, tile
+ * order, grid), touches no device, allocates and launches nothing, dereferences no pointer (pointer
+ * values matter only for their alignment), and writes what would be launched to plan[0..TI_PLAN_INTS):
+ *   [0] configuration index  [1] K splits  [2] k-tiles per split  [3] row tiles  [4] column tiles
+ *   [5] row tiles per group of the tile order  [6] grid x  [7] grid y  [8] threads per workgroup
+ *   [9] waves that split K inside a workgroup (skinny / rows4 kernels)  [10] streaming waves (rows4)
+ *   [11] bytes of split-K partial sums the launch needs
+ * Runs without a GPU.  The autotuner of the reference (kernels/utils.py:6-558) answers the same
+ * question -- which tile for which (M, N, K) -- by timing; this reports the static choice.  Used by the
+ * host-side bounds tests, which replay the kernels' address arithmetic for the planned launch.
+ */
+#define TI_PLAN_INTS 12
+int ti_gemm_plan(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk,
+                 const int8_t* B, int64_t sBb, int64_t sBn, int64_t sBk,
+                 void* C, int64_t sCb, int64_t sCm, int64_t sCn,
+                 int batch, int M, int N, int K,
+                 const void* bias, int bias_kind,
+                 const float* alpha, const float* beta,
+                 int epilogue, int out_dtype, int round_mode,
+                 int config, int static_scratch, int64_t* plan);
 
 /* ---- row kernels ------------------------------------------------------------------- */
 

@@ -25,7 +25,7 @@ TORCH_TO_DT = {torch.int8: DT_I8, torch.int32: DT_I32, torch.float32: DT_F32, to
 TORCH_TO_BIAS = {torch.int8: BIAS_I8, torch.int32: BIAS_I32, torch.float32: BIAS_F32}
 
 EXPORTS = ("ti_version", "ti_last_error", "ti_mfma_i8_probe", "ti_bmm_i8", "ti_bmm_i8_config", "ti_bmm_i8_grouped", "ti_bmm_i8_static_scratch", "ti_gemm_num_configs",
-           "ti_gemm_config_name", "ti_gemm_last_config", "ti_gemm_last_splits", "ti_layernorm_q", "ti_dq_add_layernorm_q", "ti_gelu_q", "ti_softmax_q", "ti_transpose_i8", "ti_attention_i8", "ti_quantize_per_token_absmax", "ti_kv_append_i8",
+           "ti_gemm_config_name", "ti_gemm_last_config", "ti_gemm_last_splits", "ti_gemm_plan", "ti_layernorm_q", "ti_dq_add_layernorm_q", "ti_gelu_q", "ti_softmax_q", "ti_transpose_i8", "ti_attention_i8", "ti_quantize_per_token_absmax", "ti_kv_append_i8",
            "ti_layernorm_fp", "ti_linear_i8_residual_f32", "ti_qkv_decode_i8")
 
 _lib = None
@@ -52,6 +52,8 @@ def _declare(lib):
     lib.ti_bmm_i8_grouped.argtypes = [_vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64,
                                       _int, _int, _int, _int, _vp, _int, _i64, _vp, _vp, _i64, _int, _int, _int,
                                       _int, _vp]
+    lib.ti_gemm_plan.restype = _int
+    lib.ti_gemm_plan.argtypes = bmm_args + [_int, _int, ctypes.POINTER(ctypes.c_int64)]
     lib.ti_gemm_num_configs.restype = _int
     lib.ti_gemm_num_configs.argtypes = []
     lib.ti_gemm_last_config.restype = _int

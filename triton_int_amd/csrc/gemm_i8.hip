@@ -264,9 +264,14 @@ struct TileLoader {
 // it, which drains the load pipeline once per k-tile and defeats multi-stage prefetching.  With
 // the loads invisible to that tracking, the kernel counts them itself (vmcnt retires in order).
 // M0 carries the LDS destination of a wave's 64 x 16 bytes; nothing else in these kernels uses M0.
-// The descriptor and the scalar offset handed to these helpers must come from scalar instructions
-// (kernel arguments, SALU arithmetic): the wait states a VMEM read of a VALU-written SGPR needs are
-// the compiler's job, and it does not look inside the asm.
+// Hazard the compiler cannot see: a VMEM instruction must not read an SGPR (descriptor, scalar
+// offset) within 5 wait states of a VALU instruction writing it (v_readfirstlane, the tail of a
+// uniform division), or it reads the register's previous contents -- and the scalar offset is added
+// AFTER the descriptor's range check, so a stale one addresses base + garbage.  The compiler inserts
+// those wait states for instructions it emits itself, not for the text of an asm block, so the
+// helpers carry them: s_mov m0 (1) + s_nop 3 (4) = 5 wait states between whatever precedes the block
+// and the load, wherever the operands come from.  (The s_nop also covers the one wait state a
+// buffer load to LDS needs after a write of M0.)
 __device__ __forceinline__ v4i make_rsrc(const void* base, int bytes) {
   const uint64_t a = (uint64_t)base;
   v4i r;
@@ -278,7 +283,7 @@ __device__ __forceinline__ v4i make_rsrc(const void* base, int bytes) {
 }
 
 __device__ __forceinline__ void dma16_to_lds(v4i rsrc, int voff, int soff, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                :
                : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
                : "memory");
@@ -287,7 +292,7 @@ __device__ __forceinline__ void dma16_to_lds(v4i rsrc, int voff, int soff, unsig
 // the same, non-temporal, for data that is read exactly once (the decode kernel's weight stream:
 // 7 % shorter launches than with the default cache policy)
 __device__ __forceinline__ void dma16_to_lds_stream(v4i rsrc, int voff, int soff, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen nt lds"
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tbuffer_load_dwordx4 %1, %2, %3 offen nt lds"
                :
                : "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff)
                : "memory");
@@ -1751,12 +1756,17 @@ __global__ __launch_bounds__(512, UU ? 2 : 4) void gemm_skinny_kernel(GemmParams
   if ((p.K & 63) && kpart == 0) {
     const int k0 = KSF * 64;
     const bool ok = k0 + c4 * 16 < p.K;  // K is a multiple of 16: a chunk is all in or all out
+    // a lane whose chunk lies past K reads the first 16 bytes of its row instead (the row pointers
+    // already include the lane's chunk offset c4 * 16: without taking it back, a K below 64 would
+    // put that read up to 48 bytes past the end of the row, and for the last row of the last batch
+    // entry past the end of the operand)
+    const int tail_off = ok ? k0 : -c4 * 16;
     v4i x1[MBMAX];
 #pragma unroll
-    for (int mb = 0; mb < MBMAX; ++mb) x1[mb] = *(const v4i*)(xrow[mb] + (ok ? k0 : 0));
+    for (int mb = 0; mb < MBMAX; ++mb) x1[mb] = *(const v4i*)(xrow[mb] + tail_off);
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-      v4i w1 = *(const v4i*)(wrow[g] + (ok ? k0 : 0));
+      v4i w1 = *(const v4i*)(wrow[g] + tail_off);
       if (!ok) w1 = (v4i){0, 0, 0, 0};
 #pragma unroll
       for (int mb = 0; mb < MBMAX; ++mb)
@@ -1965,11 +1975,9 @@ __global__ __launch_bounds__((R4_NW + 1) * 64) void gemm_rows4_kernel(GemmParams
     auto issue_job = [&](int j) {
       const bool real = j < njobs;
       const int cm = real ? j / nu : 0, ui = real ? j - cm * nu : 0;
-      // uniform; says so to the compiler.  The copy makes the register the loads read one that a scalar
-      // instruction wrote: a VMEM instruction must not read an SGPR within 5 wait states of a VALU
-      // instruction (v_readfirstlane) writing it, and the compiler does not see the loads inside the asm.
-      int k0 = __builtin_amdgcn_readfirstlane((kpart + cm * KS) * R4_KC);
-      asm volatile("s_mov_b32 %0, %1" : "=s"(k0) : "s"(k0));
+      // uniform; says so to the compiler (the load helper keeps the wait states a VMEM read of this
+      // VALU-written register needs)
+      const int k0 = __builtin_amdgcn_readfirstlane((kpart + cm * KS) * R4_KC);
       const int row0 = (u_first + ui * NSLOT) * R4_RG;
       const bool in = real && k0 + kl < p.K;
       const unsigned dst = ring + (j % NST) * STAGE;
@@ -2160,7 +2168,9 @@ static bool stream_eligible(const GemmParams& p) {
   if (p.sCn != 1 || p.sCm < p.N || p.sCb < 0) return false;
   const int oc = out_class(p.out_dtype);
   const int esz = oc == OUT8 ? 1 : (oc == OUT32 ? 4 : 2);
-  if (((int64_t)p.M * p.sCm + p.N) * esz >= ((int64_t)1 << 31)) return false;
+  // 32-bit store offsets, including those of the rows a ragged last tile computes past M before the
+  // range check drops them: (first row of the tile + row inside it) * pitch must not wrap back into range
+  if (((int64_t)(p.M + 512) * p.sCm + p.N) * esz >= ((int64_t)1 << 31)) return false;
   if ((uintptr_t)p.C % esz) return false;
   if (oc == OUT8 && ((p.N & 15) || (p.sCm & 15) || (p.sCb & 15) || ((uintptr_t)p.C & 15))) return false;
   return true;
@@ -2426,19 +2436,31 @@ static int sk_static_scratch(hipStream_t stream, int** partial, int** counter) {
   return TI_OK;
 }
 
+// What run() launches for a problem: filled instead of launching when run() is given one (ti_gemm_plan).
+struct LaunchPlan {
+  int config = -1, splits = 1, kt_split = 0, tiles_m = 0, tiles_n = 0, group_m = 1;
+  unsigned grid_x = 0, grid_y = 0;
+  int threads = 0, ksplit = 1, nwa = 0;
+  int64_t partial_bytes = 0;  // split-K partial sums the launch needs
+};
+
 // `config`: bits 0..7 the configuration (0xff or a negative value: choose), bits 8..15 the number of
 // K splits to use with a wave-specialised configuration (0: choose).
 // static_scratch: split-K launches use the fixed device array instead of the allocated workspace, and a
 // launch whose partial sums do not fit it is refused (nothing is allocated or freed on this path).
-static int run(GemmParams p, int config, hipStream_t stream, bool static_scratch = false) {
+// dry: every decision is taken as for a launch (same code), but no device is touched, nothing is
+// allocated or launched, and *dry receives the launch's configuration and grid.
+static int run(GemmParams p, int config, hipStream_t stream, bool static_scratch = false, LaunchPlan* dry = nullptr) {
   g_last_splits = 1;
   int want_splits = config < 0 ? 0 : (config >> 8) & 0xff;
   if (config >= 0) config = (config & 0xff) == 0xff ? -1 : (config & 0xff);
   int rc = validate(p);
   if (rc != TI_OK) return rc;
   if (p.batch == 0 || p.M == 0 || p.N == 0) return TI_OK;
-  rc = check_device();
-  if (rc != TI_OK) return rc;
+  if (!dry) {
+    rc = check_device();
+    if (rc != TI_OK) return rc;
+  }
   if (!p.bias) p.bias_kind = TI_BIAS_NONE;
   // the fast kernels quantise to int8 with round-half-even only; the truncating test switch runs
   // on the gather kernel
@@ -2496,6 +2518,11 @@ static int run(GemmParams p, int config, hipStream_t stream, bool static_scratch
     if (nwa < 8 && per > nwa) return fail(TI_E_COMBO, "config %s: %d units per workgroup need more than %d waves", k.name, per, nwa);
     g_last_config = config;
     g_last_splits = p.ksplit;
+    if (dry) {
+      dry->config = config; dry->grid_x = (unsigned)blocks; dry->grid_y = (unsigned)p.batch; dry->threads = k.threads;
+      dry->ksplit = p.ksplit; dry->nwa = nwa;
+      return TI_OK;
+    }
     rows4_kernel(out_class(p.out_dtype), nwa)<<<dim3((unsigned)blocks, (unsigned)p.batch), dim3(k.threads), 0, stream>>>(p);
     return launch_status(k.name);
   }
@@ -2512,6 +2539,10 @@ static int run(GemmParams p, int config, hipStream_t stream, bool static_scratch
     const int per_block = 8 / ksplit;
     dim3 grid((unsigned)(((p.N + k.bn - 1) / k.bn + per_block - 1) / per_block), (unsigned)p.batch, 1);
     g_last_config = config;
+    if (dry) {
+      dry->config = config; dry->grid_x = grid.x; dry->grid_y = grid.y; dry->threads = k.threads; dry->ksplit = ksplit;
+      return TI_OK;
+    }
     k.fn[out_class(p.out_dtype)]<<<grid, dim3(k.threads), 0, stream>>>(p);
     return launch_status(k.name);
   }
@@ -2534,13 +2565,15 @@ static int run(GemmParams p, int config, hipStream_t stream, bool static_scratch
         return fail(TI_E_SHAPE, "%d K splits of %lld tiles need %zu bytes of partial sums: more than the %zu bytes of static scratch "
                     "(use ti_bmm_i8, which allocates its workspace)", splits, (long long)tiles, (size_t)tiles * splits * item_bytes,
                     SK_STATIC_PARTIAL_BYTES);
-      rc = sk_static_scratch(stream, &p.sk_partial, &p.sk_counter);
-      if (rc != TI_OK) return rc;
+      if (!dry) {
+        rc = sk_static_scratch(stream, &p.sk_partial, &p.sk_counter);
+        if (rc != TI_OK) return rc;
+      }
     } else if (splits > 1 && ((size_t)tiles * k.ws_waves > SK_COUNTER_INTS || (size_t)tiles * splits * item_bytes > SK_MAX_PARTIAL_BYTES)) {
       if (want_splits) return fail(TI_E_SHAPE, "%d splits of %lld tiles exceed the split-K workspace", splits, (long long)tiles);
       splits = 1;
     }
-    if (splits > 1 && !static_scratch) {
+    if (splits > 1 && !static_scratch && !dry) {
       hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
       (void)hipStreamIsCapturing(stream, &cap);
       rc = sk_workspace(stream, (size_t)tiles * splits * item_bytes, cap == hipStreamCaptureStatusNone, &p.sk_partial, &p.sk_counter);
@@ -2549,8 +2582,13 @@ static int run(GemmParams p, int config, hipStream_t stream, bool static_scratch
       else if (rc != TI_OK) return rc;
     }
     p.splits = splits;
+    if (dry && splits > 1) dry->partial_bytes = (int64_t)((size_t)tiles * splits * item_bytes);
   }
   g_last_splits = p.splits;
+  if (dry) {
+    dry->config = config; dry->splits = p.splits; dry->kt_split = p.kt_split; dry->tiles_m = p.tiles_m; dry->tiles_n = p.tiles_n;
+    dry->group_m = p.group_m; dry->threads = k.threads;
+  }
   if (k.stream_occ) {
     const int64_t items = (int64_t)p.tiles_m * p.tiles_n * p.batch * p.splits;
     if (items > 0x7fffffff) return fail(TI_E_SHAPE, "too many tiles");
@@ -2559,10 +2597,18 @@ static int run(GemmParams p, int config, hipStream_t stream, bool static_scratch
     // workgroups without an item return at once)
     int64_t g = items < 256 * k.stream_occ ? items : 256 * k.stream_occ;
     if (g >= 8) g = (g + 7) & ~(int64_t)7;
+    if (dry) {
+      dry->grid_x = (unsigned)g; dry->grid_y = 1;
+      return TI_OK;
+    }
     k.fn[out_class(p.out_dtype)]<<<dim3((unsigned)g), dim3(k.threads), 0, stream>>>(p);
     return launch_status(k.name);
   }
   dim3 grid((unsigned)(p.tiles_m * p.tiles_n), (unsigned)p.batch, 1);
+  if (dry) {
+    dry->grid_x = grid.x; dry->grid_y = grid.y;
+    return TI_OK;
+  }
   k.fn[out_class(p.out_dtype)]<<<grid, dim3(k.threads), 0, stream>>>(p);
   return launch_status(k.name);
 }
@@ -2743,6 +2789,33 @@ int ti_linear_i8_residual_f32(const int8_t* A, int64_t lda, const int8_t* W, int
   return ti::run_with_residual(p, residual, ldr, (hipStream_t)stream);
 }
 
+
+int ti_gemm_plan(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk, const int8_t* B, int64_t sBb, int64_t sBn,
+                 int64_t sBk, void* C, int64_t sCb, int64_t sCm, int64_t sCn, int batch, int M, int N, int K,
+                 const void* bias, int bias_kind, const float* alpha, const float* beta, int epilogue, int out_dtype,
+                 int round_mode, int config, int static_scratch, int64_t* plan) {
+  if (!plan) return ti::fail(TI_E_NULL, "plan is NULL");
+  ti::GemmParams p;
+  p.A = A; p.B = B; p.C = C;
+  p.sAb = sAb; p.sAm = sAm; p.sAk = sAk;
+  p.sBb = sBb; p.sBn = sBn; p.sBk = sBk;
+  p.sCb = sCb; p.sCm = sCm; p.sCn = sCn;
+  p.batch = batch; p.M = M; p.N = N; p.K = K;
+  p.bias = bias; p.bias_kind = bias_kind;
+  p.alpha = alpha; p.beta = beta;
+  p.epilogue = epilogue; p.out_dtype = out_dtype; p.round_mode = round_mode;
+  p.tiles_m = p.tiles_n = 0; p.group_m = 1; p.ksplit = 1;
+  p.bias_bs = 0; p.scale_bs = 0;
+  p.resid = nullptr; p.resid_rs = 0;
+  p.kv_k = p.kv_vt = nullptr; p.kv_k_hs = p.kv_vt_rs = 0; p.kv_D = 1;
+  p.splits = 1; p.kt_split = 0; p.sk_partial = p.sk_counter = nullptr;
+  ti::LaunchPlan lp;
+  const int rc = ti::run(p, config, nullptr, static_scratch != 0, &lp);
+  const int64_t out[TI_PLAN_INTS] = {lp.config, lp.splits, lp.kt_split, lp.tiles_m, lp.tiles_n, lp.group_m, (int64_t)lp.grid_x,
+                                     (int64_t)lp.grid_y, lp.threads, lp.ksplit, lp.nwa, lp.partial_bytes};
+  for (int i = 0; i < TI_PLAN_INTS; ++i) plan[i] = out[i];
+  return rc;
+}
 
 int ti_gemm_num_configs(void) { return ti::g_num_configs; }
 
