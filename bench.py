@@ -23,18 +23,39 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 METRIC = "int8 GEMM TOPS (% MFMA peak), LN/GELU GB/s, W8A8 OPT-13B layer ms"
-# Bytes that crossed the L2 <-> fabric boundary per launch of a kernel on this workload (average over
-# the launches of one step), from rocprofv3 FETCH_SIZE and WRITE_SIZE passes scaled by the same
-# counters' readings for a 256 MiB device copy (x2.0 and x1.0); see profiles/.
-MEASURED_TRAFFIC_BYTES = {
-    "ws_256x128x128_w2x2_s1_p3_l4/int8": (2.0 * 52606 + 1.0 * 14816) * 1024,
+# Bytes that crossed the L2 <-> fabric boundary per launch of the dominant kernel on this workload come from
+# rocprofv3 FETCH_SIZE / WRITE_SIZE passes taken outside bench.py; their summary under profiles/ holds the
+# readings (KiB per dispatch) and the factors that scale them (from a 256 MiB device copy).  bench.py reads the
+# figure from that file's table row, so it is as fresh as the file and cannot drift from it.
+TRAFFIC_PROFILE = {
+    "ws_256x128x128_w2x2_s1_p3_l4/int8": ("profiles/gemm_ws_opt67b_linear_set_counters.md", "average of the 5 launches of a step"),
 }
-# where that reading comes from: the summary file and what the kernel's tile order was when it was
-# taken (the figure is only as fresh as that file; bench.py does not re-measure it)
-MEASURED_TRAFFIC_SOURCE = {
-    "ws_256x128x128_w2x2_s1_p3_l4/int8": "profiles/gemm_ws_opt67b_linear_set_counters.md (FETCH_SIZE x2.0 + WRITE_SIZE x1.0, KiB per "
-                                         "dispatch averaged over the 5 launches of a step)",
-}
+
+
+def traffic_from_profile(kernel):
+    """(bytes per launch, source description) for `kernel`, or (None, None): parses the row
+    '| <label> | FETCH_SIZE KiB | .. | WRITE_SIZE KiB = .. |' and the two 'factor' figures of the summary."""
+    import re
+
+    if kernel not in TRAFFIC_PROFILE:
+        return None, None
+    rel, label = TRAFFIC_PROFILE[kernel]
+    try:
+        text = open(os.path.join(ROOT, rel)).read()
+    except OSError:
+        return None, None
+    num = r"(\d[\d ]*(?:\.\d+)?)"
+    ff = re.search(r"FETCH_SIZE reads[^\n]*?factor " + num, text)
+    wf = re.search(r"WRITE_SIZE reads[^\n]*?factor " + num, text)
+    row = re.search(r"\|\s*" + re.escape(label) + r"\s*\|\s*" + num + r"\s*\|[^|]*\|\s*" + num + r"\s*KiB", text)
+    if not (ff and wf and row):
+        return None, None
+    val = lambda m, i=1: float(m.group(i).replace(" ", ""))
+    fetch_kib, write_kib = val(row, 1), val(row, 2)
+    total = (val(ff) * fetch_kib + val(wf) * write_kib) * 1024
+    return total, f"{rel}, row '{label}': FETCH_SIZE {fetch_kib:.0f} KiB x {val(ff)} + WRITE_SIZE {write_kib:.0f} KiB x {val(wf)}"
+
+
 INT8_PEAK_TOPS = 5000.0   # MI355X dense INT8 MFMA, published
 HBM_PEAK_GBPS = 8000.0    # MI355X HBM3E, published
 
@@ -352,33 +373,55 @@ def extras(torch, dev):
     return out
 
 
-def m_sweep(torch, dev, N, K, lib):
+def m_sweep(torch, dev, N, K, lib, full=True):
     """The reference's own benchmark (kernels/linear.py:960-1070): int8 x int8 -> fp32 linear with an
-    fp32 bias over M, weights [N, K]; operands made like the reference's (`randn(fp16).to(int8)`),
-    per-launch event timing, quantiles 0.5 / 0.2 / 0.8 as its `do_bench(quantiles=...)` call."""
+    fp32 bias over M in {32, 64, 128, 256} and 1024 * {1..16}, weights [N, K] = [6848, 10240]; operands made
+    like the reference's (`randn(fp16).to(int8)`: almost all bytes are 0, +-1, +-2, so the chip holds a much
+    higher clock than on uniform int8), per-launch event timing, quantiles 0.5 / 0.2 / 0.8 as its
+    `do_bench(quantiles=...)` call.  Its "triton-i8-fp16" / "-bf16" legs (bias and output in that dtype,
+    :1015-1050) are timed beside the fp32 one, and one extra leg repeats the fp32 case on uniform int8
+    operands (the distribution every other figure of this benchmark uses)."""
     from triton_int_amd.kernels import linear
 
     out = {}
     b = torch.randn((N, K), device=dev, dtype=torch.float16).to(torch.int8)
-    bias = torch.randn(N, device=dev)
+    b_uni = torch.randint(-127, 128, (N, K), dtype=torch.int8, device=dev)
+    biases = {"f32": torch.randn(N, device=dev)}
+    if full:
+        biases["f16"] = biases["f32"].half()
+        biases["bf16"] = biases["f32"].bfloat16()
     one = torch.tensor(1.0, device=dev)
-    for M in (32, 64, 128, 256, 1024, 2048, 4096, 8192, 16384):
-        a = torch.randn((M, K), device=dev, dtype=torch.float16).to(torch.int8)
+    ms_list = (32, 64, 128, 256) + tuple(1024 * i for i in range(1, 17)) if full else (32, 64, 128, 256, 1024, 2048, 4096, 8192, 16384)
+
+    def timed(a, w, bias):
         for _ in range(3):
-            linear.linear_a8_w8_bfp32_ofp32(a, b, bias, one, one)
+            linear.linear_a8_w8_bfp32_ofp32(a, w, bias, one, one)
         reps = 20
         ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
         for s_, e_ in ev:
             s_.record()
-            linear.linear_a8_w8_bfp32_ofp32(a, b, bias, one, one)
+            linear.linear_a8_w8_bfp32_ofp32(a, w, bias, one, one)
             e_.record()
         torch.cuda.synchronize()
         ts = sorted(s_.elapsed_time(e_) for s_, e_ in ev)
-        p50 = ts[len(ts) // 2]
-        out[f"M{M}"] = {"ms_p50_p20_p80": [p50, ts[len(ts) // 5], ts[4 * len(ts) // 5]],
-                        "TOPS": 2.0 * M * N * K / p50 / 1e9,
-                        "kernel": lib.ti_gemm_config_name(lib.ti_gemm_last_config()).decode(),
-                        "k_splits": lib.ti_gemm_last_splits()}
+        return ts[len(ts) // 2], ts[len(ts) // 5], ts[4 * len(ts) // 5]
+
+    for M in ms_list:
+        a = torch.randn((M, K), device=dev, dtype=torch.float16).to(torch.int8)
+        p50, p20, p80 = timed(a, b, biases["f32"])
+        rec = {"ms_p50_p20_p80": [p50, p20, p80], "TOPS": 2.0 * M * N * K / p50 / 1e9,
+               "kernel": lib.ti_gemm_config_name(lib.ti_gemm_last_config()).decode(), "k_splits": lib.ti_gemm_last_splits()}
+        for name in ("f16", "bf16"):
+            if name in biases:
+                q50, _, _ = timed(a, b, biases[name])
+                rec[f"ms_p50_{name}"] = q50
+                rec[f"TOPS_{name}"] = 2.0 * M * N * K / q50 / 1e9
+        if full:
+            au = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=dev)
+            u50, _, _ = timed(au, b_uni, biases["f32"])
+            rec["ms_p50_uniform_int8"] = u50
+            rec["TOPS_uniform_int8"] = 2.0 * M * N * K / u50 / 1e9
+        out[f"M{M}"] = rec
     return out
 
 
@@ -501,6 +544,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU emulation baseline")
     ap.add_argument("--no-extra", action="store_true", help="skip the row-kernel / BMM extras")
+    ap.add_argument("--qkv-only", type=int, default=0, metavar="N",
+                    help="run the q/k/v projections of the linear set N times as three launches and N times as one "
+                         "grouped launch, print times and held clocks, and exit: the program profiled for the "
+                         "grouped-launch counter summary")
     ap.add_argument("--decode-gemm-only", action="store_true",
                     help="run 24 launches of the M=16 decode GEMM 20480 x 5120 (int8 out, weights rotated through "
                          "6 matrices) and exit: the program profiled for the decode GEMM counter summary")
@@ -530,6 +577,51 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.qkv_only:
+        # q/k/v of the linear set (3 x 2048 x 4096 x 4096, int8 out) as three launches and as one grouped launch,
+        # each looped `--qkv-only` times with the shader clock sampled meanwhile; prints one JSON line
+        import glob
+        import threading
+
+        from triton_int_amd.kernels import linear
+
+        xq = torch.randint(-127, 128, (2048, 4096), dtype=torch.int8, device=dev)
+        w3 = torch.randint(-127, 128, (3 * 4096, 4096), dtype=torch.int8, device=dev)
+        b3 = torch.randint(-127, 128, (3 * 4096,), dtype=torch.int8, device=dev)
+        al3, be3 = torch.rand(3, device=dev) * 9e-3 + 1e-3, torch.rand(3, device=dev) * 9e-3 + 1e-3
+        o3 = torch.empty((2048, 3 * 4096), dtype=torch.int8, device=dev)
+        outs = [torch.empty((2048, 4096), dtype=torch.int8, device=dev) for _ in range(3)]
+        ws = [w3[i * 4096:(i + 1) * 4096] for i in range(3)]
+        bs = [b3[i * 4096:(i + 1) * 4096] for i in range(3)]
+
+        def three():
+            for i in range(3):
+                linear.linear_a8_w8_b8_o8(xq, ws[i], bs[i], al3[i], be3[i], out=outs[i])
+
+        def grouped():
+            linear.linear_group_a8_w8_b8_o8(xq, w3, b3, al3, be3, 3, out=o3)
+
+        sclk_file = _find_sclk_file(torch, glob)
+        res = {}
+        for name, fn in (("three_launches", three), ("grouped_launch", grouped), ("three_launches_again", three)):
+            clocks, on = [], {"v": True}
+
+            def sample():
+                while on["v"]:
+                    mhz = _read_sclk_mhz(sclk_file)
+                    if mhz:
+                        clocks.append(mhz)
+                    time.sleep(0.002)
+
+            th = threading.Thread(target=sample)
+            th.start()
+            ms = time_region(torch, fn, args.qkv_only, 5)
+            on["v"] = False
+            th.join()
+            res[name] = {"ms": ms, "TOPS": 3 * 2.0 * 2048 * 4096 * 4096 / ms / 1e9,
+                         "sclk_mhz_median": sorted(clocks)[len(clocks) // 2] if clocks else None, "sclk_samples": len(clocks)}
+        print(json.dumps({"qkv_2048x3x4096x4096": res}))
+        return
     if args.decode_gemm_only:
         from triton_int_amd.kernels import linear
 
@@ -619,11 +711,31 @@ def main():
         step()
     torch.cuda.synchronize()
     events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    # the shader clock the chip holds during the timed steps: the driver's sysfs file read from a thread
+    # (in-process, no child; the region is short, so the thread reads back to back)
+    import glob
+    import threading
+
+    sclk_file, sclk_samples, sampling = _find_sclk_file(torch, glob), [], {"on": True}
+
+    def sample_sclk():
+        while sampling["on"] and len(sclk_samples) < 400:
+            mhz = _read_sclk_mhz(sclk_file)
+            if mhz:
+                sclk_samples.append(mhz)
+            time.sleep(0.0005)
+
+    th = threading.Thread(target=sample_sclk)
+    if sclk_file:
+        th.start()
     t0 = time.perf_counter()
     for i in range(args.steps):
         step(events[i])
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
+    sampling["on"] = False
+    if sclk_file:
+        th.join()
     ms_per_step = wall * 1e3 / args.steps
     dom_ms = sum(a.elapsed_time(b) for a, b in events) / args.steps  # per step, all launches of the dominant kernel
     # device time of whole steps: start event of step i to start event of step i+1
@@ -662,12 +774,13 @@ def main():
             "peak": INT8_PEAK_TOPS,
             "unit": "TFLOP/s",
             "frac": achieved / INT8_PEAK_TOPS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get(dominant),
-            "traffic_source": MEASURED_TRAFFIC_SOURCE.get(dominant),
+            "traffic": traffic_from_profile(dominant)[0],
+            "traffic_source": traffic_from_profile(dominant)[1],
             "algorithmic_bytes": sum(x.numel() + m.weight.numel() + x.shape[0] * m.weight.shape[0]
                                      for _, m, x, _ in groups[dominant]) / n_dom,
             "launches_per_step": n_dom,
             "avg_launch_us": dom_ms * 1e3 / n_dom,
+            "sclk_mhz_during_timed_steps": (sorted(sclk_samples)[len(sclk_samples) // 2] if sclk_samples else None),
             "ops_per_launch": dom_ops / n_dom,
         },
     }
@@ -680,7 +793,7 @@ def main():
         result["extra"] = extras(torch, dev)
         result["extra"]["attention_i8_fused_vs_chain_40x2048x2048"] = attention_mismatch(torch, dev)
         result["extra"]["m_sweep_K10240_N6848"] = m_sweep(torch, dev, 6848, 10240, lib)
-        result["extra"]["m_sweep_K5120_N5120"] = m_sweep(torch, dev, 5120, 5120, lib)
+        result["extra"]["m_sweep_K5120_N5120"] = m_sweep(torch, dev, 5120, 5120, lib, full=False)
         result["extra"]["opt13b_decoder_layer"] = decoder_layer_ms(torch, dev)
         result["extra"]["sustained_fc2_2048x4096x16384"] = sustained_clock(torch, dev)
     if not args.no_cpu:

@@ -57,7 +57,10 @@ enum ti_epilogue {
 };
 
 enum ti_dtype { TI_I8 = 0, TI_I32 = 1, TI_F32 = 2, TI_F16 = 3, TI_BF16 = 4 };
-enum ti_bias { TI_BIAS_NONE = 0, TI_BIAS_I8 = 1, TI_BIAS_I32 = 2, TI_BIAS_F32 = 3 };
+/* TI_BIAS_F16 / TI_BIAS_BF16: TI_EPI_SCALE_F only; the elements are widened to fp32 exactly, i.e. the
+ * result is that of passing bias.float() (the reference's launcher takes the bias in the output's
+ * dtype, kernels/linear.py:830-832, and its kernel widens it on load, :786-790). */
+enum ti_bias { TI_BIAS_NONE = 0, TI_BIAS_I8 = 1, TI_BIAS_I32 = 2, TI_BIAS_F32 = 3, TI_BIAS_F16 = 4, TI_BIAS_BF16 = 5 };
 enum ti_round { TI_ROUND_RNE_CLAMP = 0, TI_ROUND_TRUNC = 1 };
 
 enum ti_status {
@@ -164,9 +167,10 @@ int ti_bmm_i8_grouped(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk,
  * its ticket counters and int32 partial sums: in a fixed array in the library's device image
  * (16384 counters + 32 MiB of partial sums, held by every GPU the library runs on until the process
  * ends) instead of the per-stream workspace ti_bmm_i8 allocates.  The call allocates and frees
- * nothing, on the host side of the device or through any library.  A launch whose partial sums
- * would not fit (tiles x splits x tile bytes > 32 MiB, or tiles x 4 > 16384) returns TI_E_SHAPE and
- * launches nothing; launches that do not split K use no scratch and always fit.  All calls on one
+ * nothing, on the host side of the device or through any library.  A K split the caller forces
+ * (bits 8..15 of config) whose partial sums would not fit (tiles x splits x tile bytes > 32 MiB, or
+ * tiles x 4 > 16384) returns TI_E_SHAPE and launches nothing; a split the library would choose itself
+ * gives way to the unsplit launch in that case (same result; it uses no scratch and always fits).  All calls on one
  * GPU share that GPU's array: two calls that may run at the same time on one GPU (different
  * streams, different host threads) race on it and must be serialised by the caller.  Kernels leave
  * the counters at zero; the partial sums are overwritten before they are read.
@@ -179,6 +183,17 @@ int ti_bmm_i8_static_scratch(const int8_t* A, int64_t sAb, int64_t sAm, int64_t 
                              const float* alpha, const float* beta,
                              int epilogue, int out_dtype, int round_mode,
                              int config, void* stream);
+/*
+ * Frees the split-K workspaces (ticket counters + partial sums, including blocks a workspace has outgrown)
+ * that ti_bmm_i8* allocated on the current device for `stream`, or for every stream when all_streams != 0,
+ * after waiting for the work queued on those streams.  *freed_bytes (host, may be NULL) receives the bytes
+ * of the current blocks released.  A caller that creates streams per request calls this before destroying
+ * a stream; otherwise each stream that ever ran a split-K launch keeps up to 96 MiB until the process ends.
+ * A graph that captured a split-K launch on such a stream must not be replayed afterwards.  The next
+ * split-K launch allocates a new workspace.  No counterpart in the reference (Triton's autotuner
+ * allocates and frees through torch).
+ */
+int ti_release_workspaces(void* stream, int all_streams, int64_t* freed_bytes);
 int ti_gemm_num_configs(void);
 const char* ti_gemm_config_name(int config);
 /* Index of the configuration the calling thread's most recent ti_bmm_i8* launch used (-1 if
@@ -267,7 +282,7 @@ int ti_gelu_q(const float* x, const float* scale, int8_t* y, int64_t n,
  *     e_j = exp2(fma(float(x_j), s2, -(float(mx) * s2)))
  *     S   = sum_j round_half_even(e_j * 2^23)              an integer: exact in any order
  *     y_j = round_half_even(e_j * (127 * 2^23 / float(S)))     float(S) correctly rounded, IEEE division
- * scale is a host float (score scale), >= 0.  causal_q_len > 0: rows come in groups of that many query
+ * scale is a host float (score scale), 0 <= scale <= 64 (TI_E_COMBO otherwise).  causal_q_len > 0: rows come in groups of that many query
  * positions, position i attends to columns 0 .. i + (cols - causal_q_len); 0 = no mask.
  * cols <= 8192.  Row strides in elements, unit column stride.
  */
@@ -332,7 +347,7 @@ int ti_kv_append_i8(const int8_t* k_src, int64_t k_src_row_stride, const int8_t*
  *     out    = q8(pv_alpha * (probs . v))                  (bmm_s8t_s8n_s8t again, b = V^T)
  * q [batch, S, D], k [batch, T, D], vt [batch, D, T] (V^T, as the P.V BMM takes it), out
  * [batch, S, D]; int8, unit stride along the last dimension, batch and row strides in elements
- * (all multiples of 16, like the pointers); D = 128; T a multiple of 16; score_scale > 0.
+ * (all multiples of 16, like the pointers); D = 128; T a multiple of 16; 0 < score_scale <= 64.
  * The scalars are host floats.  The int8 scores are the BMM's and the probabilities ti_softmax_q's
  * bit for bit (a row's exponentials are summed as integers, so the order in which the keys are
  * visited does not matter): the output equals the three-launch chain's exactly.

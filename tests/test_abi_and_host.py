@@ -210,5 +210,9 @@ def test_c_abi_status_codes_with_raw_ctypes():
     assert "y / ln_out_f32" in err()
     assert lib.ti_softmax_q(P, 16, 0.1, P, 16, 4, 16, 32, None) == TI_E_SHAPE               # causal_q_len > cols
     assert lib.ti_softmax_q(0, 16, 0.1, P, 16, 4, 16, 0, None) == TI_E_NULL
+    assert lib.ti_softmax_q(P, 16, 100.0, P, 16, 4, 16, 0, None) == TI_E_COMBO and "scale" in err()   # beyond the exact range
+    assert lib.ti_softmax_q(P, 16, -0.1, P, 16, 4, 16, 0, None) == TI_E_COMBO
+    assert lib.ti_attention_i8(P, 2048, 128, P, 2048, 128, P, 2048, 16, P, 2048, 128, 1, 16, 16, 128, 1e-3, 100.0, 0.01, 0, None) == TI_E_COMBO
+    assert lib.ti_attention_i8(P, 2048, 128, P, 2048, 128, P, 2048, 16, P, 2048, 128, 1, 16, 16, 128, 1e-3, 0.0, 0.01, 0, None) == TI_E_COMBO
     assert lib.ti_qkv_decode_i8(P, 64, P, 64, 0, P, P, P, 64, 32, 64, 2048, P, 64, P, 64, 16, None) == TI_E_COMBO  # M > 16
     assert lib.ti_mfma_i8_probe(-1, 0, None, None) == TI_E_SHAPE

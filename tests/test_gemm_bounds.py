@@ -122,3 +122,20 @@ def test_pitched_operands_and_outputs(lib):
     pl = G.plan_for(lib, pr, EPI_SCALE_I8, B_I8)
     assert pl.name.startswith(("mfma_", "gather", "skinny")), pl.name
     G.check_launch(pr, pl)
+
+
+def test_static_scratch_falls_back_to_the_unsplit_launch_when_an_automatic_split_does_not_fit(lib):
+    # 129 x 11264 x 32768, fp32 out: the library would split K in 3 (33 MiB of partial sums); the entry point
+    # that may not allocate has 32 MiB and runs the same problem unsplit instead of refusing it
+    pr = G.contiguous(1, 129, 11264, 32768, F32)
+    pl = G.plan_for(lib, pr, EPI_SCALE_F, B_F32)
+    assert pl.splits > 1 and pl.partial_bytes > (32 << 20), pl
+    ps = G.plan_for(lib, pr, EPI_SCALE_F, B_F32, static_scratch=1)
+    assert ps.splits == 1 and ps.partial_bytes == 0 and ps.name == pl.name
+    G.check_launch(pr, ps, store_sample=8)
+    # a split the caller forces is refused when it does not fit (status TI_E_SHAPE, message names the scratch)
+    import ctypes
+    out = (ctypes.c_int64 * 12)()
+    rc = lib.ti_gemm_plan(pr.a_base, pr.sAb, pr.sAm, 1, pr.b_base, pr.sBb, pr.sBn, 1, pr.c_base, pr.sCb, pr.sCm, 1, 1, pr.M, pr.N, pr.K,
+                          1 << 12, B_F32, 1 << 12, 1 << 12, EPI_SCALE_F, F32, 0, pl.config | (3 << 8), 1, out)
+    assert rc == -2 and "static scratch" in lib.ti_last_error().decode()

@@ -133,6 +133,13 @@ def test_all_configs_float_and_scaled_i32(shape):
         assert np.array_equal(got, want_h), f"f16 {name}"
         got = cpu(linear.linear_a8_w8_bfp32_ofp32(ga, gw, gpu(bias_f), alpha, beta, dtype=torch.bfloat16, _config=cfg))
         assert np.array_equal(got, want_b), f"bf16 {name}"
+        # a bias given in fp16 / bf16 (the reference's "triton-i8-fp16" / "-bf16" benchmark legs, kernels/linear.py:
+        # 1015-1050) sets the output dtype and is widened inside the kernel: the result is that of bias.float()
+        for tdt, odt in ((torch.float16, O.DT_F16), (torch.bfloat16, O.DT_BF16)):
+            b16 = gpu(bias_f).to(tdt)
+            want16 = O.linear_a8_w8_bfp32_ofp32(a, w, b16.float().cpu().numpy(), alpha, beta, out_dtype=odt)
+            out16 = linear.linear_a8_w8_bfp32_ofp32(ga, gw, b16, alpha, beta, _config=cfg)
+            assert out16.dtype == tdt and np.array_equal(cpu(out16), want16), f"{tdt} bias {name}"
         got = cpu(linear.linear_a8_w8_ofp32(ga, gw, alpha, _config=cfg))
         assert np.array_equal(got, want_nb), f"ofp32 {name}"
         got = cpu(linear.linear_a8_w8_b32_o32_with_scaling(ga, gw, gpu(bias_i), alpha, beta, _config=cfg))
@@ -528,6 +535,42 @@ def test_split_k_on_two_streams_and_under_graph_capture():
         graph.replay()
         torch.cuda.synchronize()
         assert np.array_equal(cpu(out), want)
+
+
+def test_split_k_workspaces_of_short_lived_streams_are_released():
+    """A caller that creates a stream per request and releases the library's workspace before dropping it
+    leaves the device's free memory where it was: 200 streams, each with a split-K launch."""
+    linear, _, _ = _kl()
+    L = _lib()
+    g = rng(6)
+    M, N, K = 128, 1024, 8192
+    a, w, b32 = rand_i8(g, M, K), rand_i8(g, N, K), g.integers(-2**20, 2**20, size=N, dtype=np.int32)
+    ga, gw, gb = gpu(a), gpu(w), gpu(b32)
+    want = O.linear_a8_w8_b32_o32(a, w, b32)
+    out = torch.empty((M, N), dtype=torch.int32, device=DEV)
+    L.release_workspaces(all_streams=True)   # what earlier tests left behind
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    for i in range(200):
+        st = torch.cuda.Stream()
+        with torch.cuda.stream(st):
+            linear.linear_a8_w8_b32_o32(ga, gw, gb, out=out)
+            assert L.lib().ti_gemm_last_splits() > 1
+            freed = L.release_workspaces()   # waits for the stream, frees its blocks
+        assert freed > 0
+        if i % 50 == 0:
+            assert np.array_equal(cpu(out), want)
+        del st
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] >= free0, "workspaces of released streams still hold device memory"
+    # without a release a stream's workspace stays (that is the documented default)
+    st = torch.cuda.Stream()
+    with torch.cuda.stream(st):
+        linear.linear_a8_w8_b32_o32(ga, gw, gb, out=out)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] < free0
+    assert L.release_workspaces(all_streams=True) > 0
+    assert np.array_equal(cpu(out), want)
 
 
 @pytest.mark.parametrize("M,N,K", [(16, 5136, 1104), (9, 400, 2048), (1, 48, 64), (13, 5120, 5120)])

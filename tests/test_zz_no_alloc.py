@@ -77,6 +77,14 @@ def test_static_scratch_rejects_what_does_not_fit_and_is_capturable():
     want = torch.empty_like(out)
     assert _call(lib.ti_bmm_i8_config, ga, gw, gbf, alpha, beta, want, L.EPI_SCALE_F, ws256) == 0
     assert torch.equal(out, want)
+    # a split the library chooses itself and that does not fit gives way to the unsplit launch: same result
+    M2, N2, K2 = 129, 11264, 32768
+    ga2, gw2, gbf2 = gpu(rand_i8(g, M2, K2)), gpu(rand_i8(g, N2, K2)), gpu(g.standard_normal(N2).astype(np.float32))
+    out2, want2 = torch.empty((M2, N2), dtype=torch.float32, device=DEV), torch.empty((M2, N2), dtype=torch.float32, device=DEV)
+    assert _call(lib.ti_bmm_i8_config, ga2, gw2, gbf2, alpha, beta, want2, L.EPI_SCALE_F, -1) == 0 and lib.ti_gemm_last_splits() > 1
+    assert _call(lib.ti_bmm_i8_static_scratch, ga2, gw2, gbf2, alpha, beta, out2, L.EPI_SCALE_F, -1) == 0 and lib.ti_gemm_last_splits() == 1
+    assert torch.equal(out2, want2)
+    del ga2, gw2, gbf2, out2, want2
     # unsplit launches use no scratch at all and are never refused for size
     assert _call(lib.ti_bmm_i8_static_scratch, ga, gw, gbf, alpha, beta, out, L.EPI_SCALE_F, -1) == 0
     assert torch.equal(out, want)

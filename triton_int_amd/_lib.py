@@ -17,15 +17,16 @@ LIB_PATH = os.path.join(_HERE, "lib", "libtriton_int_hip.so")
 # enum ti_epilogue / ti_dtype / ti_bias / ti_round
 EPI_I32, EPI_SCALE_I32, EPI_SCALE_I8, EPI_SCALE_RELU_I8, EPI_SCALE_F, EPI_GELU_I8 = range(6)
 DT_I8, DT_I32, DT_F32, DT_F16, DT_BF16 = range(5)
-BIAS_NONE, BIAS_I8, BIAS_I32, BIAS_F32 = range(4)
+BIAS_NONE, BIAS_I8, BIAS_I32, BIAS_F32, BIAS_F16, BIAS_BF16 = range(6)
 ROUND_RNE_CLAMP, ROUND_TRUNC = 0, 1
 
 TORCH_TO_DT = {torch.int8: DT_I8, torch.int32: DT_I32, torch.float32: DT_F32, torch.float16: DT_F16,
                torch.bfloat16: DT_BF16}
-TORCH_TO_BIAS = {torch.int8: BIAS_I8, torch.int32: BIAS_I32, torch.float32: BIAS_F32}
+TORCH_TO_BIAS = {torch.int8: BIAS_I8, torch.int32: BIAS_I32, torch.float32: BIAS_F32, torch.float16: BIAS_F16,
+                 torch.bfloat16: BIAS_BF16}
 
 EXPORTS = ("ti_version", "ti_last_error", "ti_mfma_i8_probe", "ti_bmm_i8", "ti_bmm_i8_config", "ti_bmm_i8_grouped", "ti_bmm_i8_static_scratch", "ti_gemm_num_configs",
-           "ti_gemm_config_name", "ti_gemm_last_config", "ti_gemm_last_splits", "ti_gemm_plan", "ti_layernorm_q", "ti_dq_add_layernorm_q", "ti_gelu_q", "ti_softmax_q", "ti_transpose_i8", "ti_attention_i8", "ti_quantize_per_token_absmax", "ti_kv_append_i8",
+           "ti_gemm_config_name", "ti_gemm_last_config", "ti_gemm_last_splits", "ti_gemm_plan", "ti_release_workspaces", "ti_layernorm_q", "ti_dq_add_layernorm_q", "ti_gelu_q", "ti_softmax_q", "ti_transpose_i8", "ti_attention_i8", "ti_quantize_per_token_absmax", "ti_kv_append_i8",
            "ti_layernorm_fp", "ti_linear_i8_residual_f32", "ti_qkv_decode_i8")
 
 _lib = None
@@ -54,6 +55,8 @@ def _declare(lib):
                                       _int, _vp]
     lib.ti_gemm_plan.restype = _int
     lib.ti_gemm_plan.argtypes = bmm_args + [_int, _int, ctypes.POINTER(ctypes.c_int64)]
+    lib.ti_release_workspaces.restype = _int
+    lib.ti_release_workspaces.argtypes = [_vp, _int, ctypes.POINTER(ctypes.c_int64)]
     lib.ti_gemm_num_configs.restype = _int
     lib.ti_gemm_num_configs.argtypes = []
     lib.ti_gemm_last_config.restype = _int
@@ -153,6 +156,7 @@ def require_cuda(*tensors) -> None:
 
 
 _scalar_cache: dict = {}
+_SCALAR_CACHE_MAX = 1024  # distinct (value, device) pairs kept; beyond it python-float scales are uploaded per call
 
 
 def scale_tensor(v, device) -> torch.Tensor:
@@ -175,5 +179,19 @@ def scale_tensor(v, device) -> torch.Tensor:
                 f"scale {float(v)!r} was first seen during HIP graph capture; pass scales as fp32 device "
                 "tensors, or run the call once before capturing")
         t = torch.tensor(float(v), dtype=torch.float32, device=device)
-        _scalar_cache[key] = t
+        # Bounded: a caller that passes a fresh python float on every call (a dynamic per-batch scale) would
+        # otherwise grow the cache without end.  Past the bound the upload is simply not kept: the launcher
+        # holds the tensor until the launch is enqueued, and the allocator hands its block only to later work
+        # of the same stream.  Dynamic scales belong in device tensors, which take no upload at all.
+        if len(_scalar_cache) < _SCALAR_CACHE_MAX:
+            _scalar_cache[key] = t
     return t
+
+
+def release_workspaces(stream=None, all_streams: bool = False) -> int:
+    """Frees the split-K workspaces the library holds for `stream` (default: torch's current stream) on the
+    current device, or for every stream; returns the bytes freed.  Waits for the streams' queued work."""
+    freed = ctypes.c_int64(0)
+    h = current_stream(torch.device("cuda", torch.cuda.current_device())) if stream is None else int(stream)
+    check(lib().ti_release_workspaces(h, 1 if all_streams else 0, ctypes.byref(freed)), "ti_release_workspaces")
+    return int(freed.value)

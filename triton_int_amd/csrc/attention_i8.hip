@@ -547,11 +547,9 @@ extern "C" int ti_attention_i8(const int8_t* q, int64_t q_batch_stride, int64_t 
                           (uintptr_t)vt_batch_stride | (uintptr_t)vt_row_stride | (uintptr_t)out_batch_stride |
                           (uintptr_t)out_row_stride;
   if (align & 15) return fail(TI_E_STRIDE, "pointers and strides must be multiples of 16 bytes");
-  // exponentials are taken against the largest possible score (127): the smallest one must stay a
-  // normal fp32 number
   const float s2 = score_scale * 1.44269504088896340736f;
-  if (!(score_scale > 0.0f) || !(s2 < 3.0e38f))
-    return fail(TI_E_COMBO, "score_scale %g is not a positive finite number", (double)score_scale);
+  if (!(score_scale > 0.0f) || !(score_scale <= SM_MAX_SCALE))
+    return fail(TI_E_COMBO, "score_scale %g outside (0, %g]: the quantised softmax is exact in that range only", (double)score_scale, (double)SM_MAX_SCALE);
   const int64_t lim32 = (int64_t)1 << 31;
   const bool few_rows = S <= 16 && T <= AD_MAXT && (int64_t)T * k_row_stride < lim32 && (int64_t)AT_D * vt_row_stride < lim32 &&
                         (int64_t)S * q_row_stride < lim32;

@@ -120,7 +120,12 @@ __device__ __forceinline__ float column_term_t(const EpiCtx& e, int n, bool gelu
   float b;
   if constexpr (KIND == TI_BIAS_I8) b = (float)((const int8_t*)base)[idx];
   else if constexpr (KIND == TI_BIAS_I32) b = (float)((const int32_t*)base)[idx];
-  else b = ((const float*)base)[idx];
+  else {
+    // the floating-point family: fp32, or fp16 / bf16 widened exactly (what bias.float() gives)
+    if (e.bias_kind == TI_BIAS_F16) b = has ? (float)((const _Float16*)base)[idx] : 0.0f;
+    else if (e.bias_kind == TI_BIAS_BF16) b = has ? __uint_as_float((unsigned)((const uint16_t*)base)[idx] << 16) : 0.0f;
+    else b = ((const float*)base)[idx];
+  }
   const float scaled = gelu ? b : b * e.beta;
   return has ? scaled : 0.0f;
 }
@@ -130,7 +135,9 @@ __device__ __forceinline__ float column_term(const EpiCtx& e, int n) {
   switch (e.bias_kind) {
     case TI_BIAS_I8: return column_term_t<TI_BIAS_I8>(e, n, gelu);
     case TI_BIAS_I32: return column_term_t<TI_BIAS_I32>(e, n, gelu);
-    case TI_BIAS_F32: return column_term_t<TI_BIAS_F32>(e, n, gelu);
+    case TI_BIAS_F32:
+    case TI_BIAS_F16:
+    case TI_BIAS_BF16: return column_term_t<TI_BIAS_F32>(e, n, gelu);
     default: return 0.0f;
   }
 }
@@ -191,7 +198,7 @@ __device__ __forceinline__ EpiCtx make_epi(const GemmParams& p, int bz) {
   e.epilogue = p.epilogue;
   e.round_mode = p.round_mode;
   e.bias_kind = p.bias ? p.bias_kind : TI_BIAS_NONE;
-  const int bias_esz = p.bias_kind == TI_BIAS_I8 ? 1 : 4;
+  const int bias_esz = p.bias_kind == TI_BIAS_I8 ? 1 : ((p.bias_kind == TI_BIAS_F16 || p.bias_kind == TI_BIAS_BF16) ? 2 : 4);
   e.bias = p.bias ? (const void*)((const char*)p.bias + (int64_t)bz * p.bias_bs * bias_esz) : nullptr;
   e.safe = (const float*)p.A;
   return e;
@@ -2334,7 +2341,8 @@ static int validate(const GemmParams& p) {
     case TI_EPI_SCALE_I8:
     case TI_EPI_SCALE_RELU_I8: ok = p.out_dtype == TI_I8 && (bk == TI_BIAS_NONE || bk == TI_BIAS_I8); break;
     case TI_EPI_SCALE_F:
-      ok = (p.out_dtype == TI_F32 || p.out_dtype == TI_F16 || p.out_dtype == TI_BF16) && (bk == TI_BIAS_NONE || bk == TI_BIAS_F32);
+      ok = (p.out_dtype == TI_F32 || p.out_dtype == TI_F16 || p.out_dtype == TI_BF16) &&
+           (bk == TI_BIAS_NONE || bk == TI_BIAS_F32 || bk == TI_BIAS_F16 || bk == TI_BIAS_BF16);
       break;
     case TI_EPI_GELU_I8: ok = p.out_dtype == TI_I8 && (bk == TI_BIAS_NONE || bk == TI_BIAS_F32); break;
     default: break;
@@ -2359,9 +2367,13 @@ static thread_local int g_last_splits = 1;
 // demand.
 constexpr size_t SK_COUNTER_INTS = 1 << 16;             // tiles x consumer waves of one launch
 constexpr size_t SK_MAX_PARTIAL_BYTES = (size_t)96 << 20;  // < 2 GiB: the kernel addresses it with 32-bit offsets
-struct SkWorkspace { int dev; hipStream_t stream; char* base; size_t partial_bytes; };
+struct SkWorkspace { int dev; hipStream_t stream; char* base; size_t partial_bytes; std::vector<char*> outgrown; };
 static std::mutex g_sk_mutex;
 static std::vector<SkWorkspace> g_sk_ws;
+
+__global__ __launch_bounds__(256) void sk_clear_counters_kernel(int* counters, int n) {
+  for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) counters[i] = 0;
+}
 
 // 0 and the pointers, or a status.  With allocate == false (the stream is being captured into a
 // graph: no allocation possible) an existing workspace that is large enough is used, else TI_E_COMBO.
@@ -2375,19 +2387,28 @@ static int sk_workspace(hipStream_t stream, size_t partial_bytes, bool allocate,
     if (e.dev == dev && e.stream == stream) w = &e;
   if (!w || w->partial_bytes < partial_bytes) {
     if (!allocate) return TI_E_COMBO;
-    // An outgrown workspace is not freed: a captured graph may hold its address.  Growing at least
-    // doubles it, so what stays behind is less than the final size.
     if (w && partial_bytes < 2 * w->partial_bytes) partial_bytes = 2 * w->partial_bytes;
     if (partial_bytes > SK_MAX_PARTIAL_BYTES) partial_bytes = SK_MAX_PARTIAL_BYTES;
     char* base = nullptr;
     const size_t bytes = SK_COUNTER_INTS * sizeof(int) + partial_bytes;
     err = hipMalloc((void**)&base, bytes);
-    if (err == hipSuccess) err = hipMemset(base, 0, SK_COUNTER_INTS * sizeof(int));
     if (err != hipSuccess) return fail((int)err, "split-K workspace of %zu bytes: %s", bytes, hipGetErrorString(err));
+    // cleared on the launch stream, so that the clear is ordered before the launch on any kind of stream
+    // (a memset on the null stream is not ordered against a non-blocking stream)
+    sk_clear_counters_kernel<<<dim3(64), dim3(256), 0, stream>>>((int*)base, (int)SK_COUNTER_INTS);
+    const int rc = launch_status("sk_clear_counters_kernel");
+    if (rc != TI_OK) {
+      (void)hipFree(base);
+      return rc;
+    }
     if (!w) {
-      g_sk_ws.push_back({dev, stream, nullptr, 0});
+      g_sk_ws.push_back({dev, stream, nullptr, 0, {}});
       w = &g_sk_ws.back();
     }
+    // The outgrown block is kept until the workspace is released: earlier launches on the stream, or a
+    // captured graph, may still use it.  Growing at least doubles the size, so the blocks kept sum to
+    // less than the current one.
+    if (w->base) w->outgrown.push_back(w->base);
     w->base = base;
     w->partial_bytes = partial_bytes;
   }
@@ -2396,6 +2417,41 @@ static int sk_workspace(hipStream_t stream, size_t partial_bytes, bool allocate,
   return TI_OK;
 }
 
+// Frees the current device's workspace of `stream` (all streams' when all != 0), outgrown blocks
+// included, after the stream's queued work has finished.  For callers that create streams per request:
+// without it every stream that ever ran a split-K launch keeps its blocks for the life of the process.
+// The caller must not replay a graph that captured a split-K launch on that stream afterwards.
+static int sk_release(hipStream_t stream, bool all, int64_t* freed_bytes) {
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return fail((int)err, "hipGetDevice: %s", hipGetErrorString(err));
+  std::vector<SkWorkspace> mine;
+  {
+    std::lock_guard<std::mutex> lock(g_sk_mutex);
+    for (size_t i = 0; i < g_sk_ws.size();) {
+      if (g_sk_ws[i].dev == dev && (all || g_sk_ws[i].stream == stream)) {
+        mine.push_back(g_sk_ws[i]);
+        g_sk_ws[i] = g_sk_ws.back();
+        g_sk_ws.pop_back();
+      } else {
+        ++i;
+      }
+    }
+  }
+  int64_t freed = 0;
+  int rc = TI_OK;
+  for (auto& w : mine) {
+    err = hipStreamSynchronize(w.stream);  // the launches that use the blocks
+    if (err != hipSuccess && rc == TI_OK) rc = fail((int)err, "hipStreamSynchronize: %s", hipGetErrorString(err));
+    if (w.base) {
+      (void)hipFree(w.base);
+      freed += (int64_t)(SK_COUNTER_INTS * sizeof(int) + w.partial_bytes);
+    }
+    for (char* b : w.outgrown) (void)hipFree(b);
+  }
+  if (freed_bytes) *freed_bytes = freed;
+  return rc;
+}
 
 // ---- split-K scratch that needs no allocation ---------------------------------------------------------
 // For callers that cannot allocate (a stream under graph capture, a serving loop that forbids it):
@@ -2409,14 +2465,12 @@ constexpr size_t SK_STATIC_INTS = SK_STATIC_COUNTER_INTS + SK_STATIC_PARTIAL_BYT
 static __device__ __align__(256) int scratch[SK_STATIC_INTS];
 static int* g_scratch_ptr[64];
 
-__global__ __launch_bounds__(256) void sk_clear_counters_kernel(int* counters, int n) {
-  for (int i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) counters[i] = 0;
-}
-
 // Device address of the calling thread's current device's copy of `scratch`.  First call on a
-// device: looks the address up and zero-fills the ticket counters with a small kernel on `stream`
-// (launches leave them at zero afterwards); no allocation, no memset node.
+// device: looks the address up.  The ticket counters need no clearing: a file-scope device array is
+// zero-initialised when the code object is loaded, and every launch leaves them at zero; so the call
+// enqueues nothing but the GEMM itself (a first call under graph capture records no extra node).
 static int sk_static_scratch(hipStream_t stream, int** partial, int** counter) {
+  (void)stream;
   int dev = 0;
   hipError_t err = hipGetDevice(&dev);
   if (err != hipSuccess) return fail((int)err, "hipGetDevice: %s", hipGetErrorString(err));
@@ -2426,9 +2480,6 @@ static int sk_static_scratch(hipStream_t stream, int** partial, int** counter) {
     int* ptr = nullptr;
     err = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
     if (err != hipSuccess || !ptr) return fail(err != hipSuccess ? (int)err : TI_E_NULL, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(err));
-    sk_clear_counters_kernel<<<dim3(16), dim3(256), 0, stream>>>(ptr, (int)SK_STATIC_COUNTER_INTS);
-    const int rc = launch_status("sk_clear_counters_kernel");
-    if (rc != TI_OK) return rc;
     g_scratch_ptr[dev] = ptr;
   }
   *counter = g_scratch_ptr[dev];
@@ -2560,11 +2611,17 @@ static int run(GemmParams p, int config, hipStream_t stream, bool static_scratch
     int splits = want_splits ? want_splits : auto_splits;
     sk_shape(kt, splits, splits, p.kt_split);
     const size_t item_bytes = (size_t)k.bm * k.bn * sizeof(int);
-    if (splits > 1 && static_scratch) {
-      if ((size_t)tiles * k.ws_waves > SK_STATIC_COUNTER_INTS || (size_t)tiles * splits * item_bytes > SK_STATIC_PARTIAL_BYTES)
+    if (splits > 1 && static_scratch &&
+        ((size_t)tiles * k.ws_waves > SK_STATIC_COUNTER_INTS || (size_t)tiles * splits * item_bytes > SK_STATIC_PARTIAL_BYTES)) {
+      // a split the caller forced is refused; one the library chose itself gives way to the unsplit launch,
+      // which needs no scratch at all (as the allocating path does when its workspace limit is exceeded)
+      if (want_splits)
         return fail(TI_E_SHAPE, "%d K splits of %lld tiles need %zu bytes of partial sums: more than the %zu bytes of static scratch "
                     "(use ti_bmm_i8, which allocates its workspace)", splits, (long long)tiles, (size_t)tiles * splits * item_bytes,
                     SK_STATIC_PARTIAL_BYTES);
+      sk_shape(kt, 1, splits, p.kt_split);
+    }
+    if (splits > 1 && static_scratch) {
       if (!dry) {
         rc = sk_static_scratch(stream, &p.sk_partial, &p.sk_counter);
         if (rc != TI_OK) return rc;
@@ -2815,6 +2872,10 @@ int ti_gemm_plan(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk, const i
                                      (int64_t)lp.grid_y, lp.threads, lp.ksplit, lp.nwa, lp.partial_bytes};
   for (int i = 0; i < TI_PLAN_INTS; ++i) plan[i] = out[i];
   return rc;
+}
+
+int ti_release_workspaces(void* stream, int all_streams, int64_t* freed_bytes) {
+  return ti::sk_release((hipStream_t)stream, all_streams != 0, freed_bytes);
 }
 
 int ti_gemm_num_configs(void) { return ti::g_num_configs; }

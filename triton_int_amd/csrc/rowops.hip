@@ -641,6 +641,7 @@ int ti_softmax_q(const int8_t* x, int64_t x_row_stride, float scale, int8_t* y, 
   if (causal_q_len > 0 && rows % causal_q_len) return ti::fail(TI_E_SHAPE, "rows %d not a multiple of causal_q_len %d", rows, causal_q_len);
   if (cols > 64 * 16 * 8) return ti::fail(TI_E_SHAPE, "softmax rows longer than 8192 are not supported");
   if (!(scale >= 0.0f)) return ti::fail(TI_E_COMBO, "the score scale must be >= 0 (the exponent is taken against the row's largest score)");
+  if (scale > ti::SM_MAX_SCALE) return ti::fail(TI_E_COMBO, "score scale %g above %g: the quantised softmax is exact up to that scale only", (double)scale, (double)ti::SM_MAX_SCALE);
   int rc = ti::check_device();
   if (rc != TI_OK) return rc;
   hipStream_t s = (hipStream_t)stream;

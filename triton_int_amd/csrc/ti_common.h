@@ -72,11 +72,17 @@ __device__ __forceinline__ float gelu_tanh_scaled(float x, float scale) {
 // agree bit for bit whatever the order in which they visit a row:
 //   mx  = the row's largest visible score (an integer: exact in any order)
 //   t   = fma(float(x), s2, c),  c = -(float(mx) * s2),  s2 = scale * log2(e)
-//   e   = exp2(t)                                      (in (0, 1], exactly 1 at the maximum)
+//   e   = exp2(t)                                      (at the maximum t is the rounding residue of
+//                                                       mx * s2, at most half an ulp of it, so e = 2^(+-d)
+//                                                       with d <= 2^-12 for scales up to SM_MAX_SCALE: the
+//                                                       steps below stay exact in that range.  Far beyond it
+//                                                       (scale ~ 1000) e * r could pass 127.5 and wrap the
+//                                                       byte; the entry points refuse such scales.)
 //   u   = rne(e * 2^23), taken from the bit pattern of 1.0f + e
 //   S   = sum of u over the row: an integer, so any order and any grouping give the same S
 //   r   = 127 * 2^23 / float(S)                        (float(S) correctly rounded, IEEE division)
 //   p   = rne(e * r): the low byte of the bit pattern of fma(e, r, 1.5 * 2^23)
+constexpr float SM_MAX_SCALE = 64.0f;           // largest score scale the entry points accept (e^64 between neighbours: one-hot)
 constexpr unsigned SM_ONE_BITS = 0x3f800000u;  // bit pattern of 1.0f: sm_unit_bits(e) - SM_ONE_BITS = u
 
 __device__ __forceinline__ unsigned sm_unit_bits(float e) { return __float_as_uint(1.0f + e); }

@@ -57,10 +57,11 @@ def linear_a8_w8_b32_o32_with_scaling(a, b, bias, scale_a, scale_b, out=None, *,
 
 def linear_a8_w8_bfp32_ofp32(a, b, bias, scale_a, scale_b, out=None, dtype=None, *, _config=-1):
     """scale_a * acc + scale_b * bias -> fp32 / fp16 / bf16; the output dtype defaults to the
-    bias dtype (reference: kernels/linear.py:819-853).  The bias is read as fp32."""
+    bias dtype (reference: kernels/linear.py:819-853).  An fp16 / bf16 bias is widened to fp32 inside the
+    kernel (no conversion launch)."""
     if dtype is None:
         dtype = out.dtype if out is not None else bias.dtype
-    if bias is not None and bias.dtype != torch.float32:
+    if bias is not None and bias.dtype not in (torch.float32, torch.float16, torch.bfloat16):
         bias = bias.to(torch.float32)
     return _linear(a, b, epilogue=L.EPI_SCALE_F, out_dtype=dtype, bias=bias, alpha=scale_a, beta=scale_b, out=out,
                    config=_config)
