@@ -549,8 +549,16 @@ def test_split_k_workspaces_of_short_lived_streams_are_released():
     want = O.linear_a8_w8_b32_o32(a, w, b32)
     out = torch.empty((M, N), dtype=torch.int32, device=DEV)
     L.release_workspaces(all_streams=True)   # what earlier tests left behind
+    # torch hands out streams from a pool it creates on first use, and a new HIP stream takes device memory of
+    # its own: create the pool before the reference reading
+    pool = [torch.cuda.Stream() for _ in range(64)]
+    for st in pool:
+        with torch.cuda.stream(st):
+            out.zero_()
     torch.cuda.synchronize()
+    del pool
     free0 = torch.cuda.mem_get_info()[0]
+    slack = 4 << 20
     for i in range(200):
         st = torch.cuda.Stream()
         with torch.cuda.stream(st):
@@ -562,13 +570,14 @@ def test_split_k_workspaces_of_short_lived_streams_are_released():
             assert np.array_equal(cpu(out), want)
         del st
     torch.cuda.synchronize()
-    assert torch.cuda.mem_get_info()[0] >= free0, "workspaces of released streams still hold device memory"
+    # 200 workspaces of about 2.3 MB each would be 460 MB
+    assert torch.cuda.mem_get_info()[0] >= free0 - slack, "workspaces of released streams still hold device memory"
     # without a release a stream's workspace stays (that is the documented default)
     st = torch.cuda.Stream()
     with torch.cuda.stream(st):
         linear.linear_a8_w8_b32_o32(ga, gw, gb, out=out)
     torch.cuda.synchronize()
-    assert torch.cuda.mem_get_info()[0] < free0
+    assert torch.cuda.mem_get_info()[0] <= free0 - (1 << 20)
     assert L.release_workspaces(all_streams=True) > 0
     assert np.array_equal(cpu(out), want)
 
