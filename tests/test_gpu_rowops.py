@@ -314,6 +314,37 @@ def test_quantize_per_token_absmax(rows, cols, dtype):
     assert np.array_equal(cpu(q2)[0], want_q) and np.array_equal(gx.float().cpu().numpy(), want_q.astype(np.float32))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_quantize_per_token_division_is_the_true_quotient(dtype):
+    """The kernel divides a row by its scale with the reciprocal part of the division hoisted out of the
+    elements; the quotients must still be the correctly rounded ones.  20 M elements per dtype against torch's own
+    element-wise steps on the GPU (true divisions), rows spanning 60 orders of magnitude, including rows whose
+    scale is outside the hoisted form's range (they take the ordinary division), an all-zero row and a row of
+    exact ties."""
+    fused = _fused()
+    rows, cols = 4096, 5120
+    gen = torch.Generator(device=DEV).manual_seed(11)
+    x = torch.randn((rows, cols), generator=gen, device=DEV, dtype=torch.float32)
+    mags = torch.logspace(-30, 30, rows, device=DEV) if dtype == torch.float32 else torch.logspace(-4, 4, rows, device=DEV)
+    x = (x * mags[:, None]).to(dtype)
+    if dtype == torch.float32:
+        x[7] = 0   # (in fp16 the clamp's 1e-8 rounds to 0 and an all-zero row is 0 / 0: not a defined case)
+    x[9] = torch.arange(cols, device=DEV).to(dtype) % 255 * 0.5 - 60.0      # k + 0.5 quotients once the scale is 1
+    x[9, 0] = 127.0
+    if dtype == torch.float32:
+        x[11] = x[11].abs() * 0 + 3.0e38
+        x[13] = torch.randn(cols, device=DEV) * 1e-38
+    # the steps of functional/quantization.py:61-67.  The scale is formed on the CPU: there torch divides by
+    # 127, as the kernel and the oracle do, where its GPU kernel for a scalar divisor multiplies by 1 / 127
+    max_val = x.abs().max(dim=-1, keepdim=True)[0].cpu()
+    max_val = (torch.clamp(max_val, min=1e-8) / 127).to(DEV)
+    want = x.clone().div_(max_val).round_().clamp_(-128, 127).to(torch.int8)  # tensor / tensor: true division
+    q, s = fused.quantize_per_token_absmax(x)
+    assert torch.equal(s, max_val)
+    bad = (q != want)
+    assert not bad.any(), (int(bad.sum()), bad.nonzero()[:4].tolist())
+
+
 @pytest.mark.parametrize("S,heads,D,T", [(16, 40, 128, 2048), (48, 4, 128, 80), (70, 3, 64, 100), (1, 2, 16, 5)])
 def test_kv_append_i8(S, heads, D, T):
     """Pure data movement: K rows into a head-major cache, V transposed into V^T columns; the

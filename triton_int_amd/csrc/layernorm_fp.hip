@@ -53,15 +53,18 @@ __device__ __forceinline__ v4u lf_pack(const float (&v)[N], float (&rounded)[N])
   return raw;
 }
 
-__device__ __forceinline__ float lf_block_sum(float v, float* red, int tid) {
+// `red` holds two sets of per-wave partial sums; consecutive reductions (counted by `k`) alternate between
+// them, so one barrier per reduction is enough (a wave that runs ahead writes the set nobody reads any more)
+__device__ __forceinline__ float lf_block_sum(float v, float* red, int tid, int& k) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-  __syncthreads();  // protect `red` from the previous use
-  if ((tid & 63) == 0) red[tid >> 6] = v;
+  float* set = red + (k & 1) * LF_WAVES;
+  ++k;
+  if ((tid & 63) == 0) set[tid >> 6] = v;
   __syncthreads();
-  float s = red[0];
+  float s = set[0];
 #pragma unroll
-  for (int w = 1; w < LF_WAVES; ++w) s += red[w];
+  for (int w = 1; w < LF_WAVES; ++w) s += set[w];
   return s;
 }
 
@@ -80,7 +83,8 @@ struct LnFpParams {
 template <typename T, int VPT>
 __global__ __launch_bounds__(LF_THREADS) void layernorm_fp_vec_kernel(LnFpParams p) {
   constexpr int N = 16 / (int)sizeof(T);
-  __shared__ float red[LF_WAVES];
+  __shared__ float red[2 * LF_WAVES];
+  int red_k = 0;
   const int tid = threadIdx.x;
   const int nvec = p.cols / N;
   const bool has_b = p.beta != nullptr;
@@ -129,7 +133,7 @@ __global__ __launch_bounds__(LF_THREADS) void layernorm_fp_vec_kernel(LnFpParams
       for (int j = 0; j < VPT; ++j)
 #pragma unroll
         for (int e = 0; e < N; ++e) s += x[j][e];  // padding vectors hold zeros
-      mean = lf_block_sum(s, red, tid) * inv_n;
+      mean = lf_block_sum(s, red, tid, red_k) * inv_n;
     }
     float m2 = 0.0f;
 #pragma unroll
@@ -142,7 +146,7 @@ __global__ __launch_bounds__(LF_THREADS) void layernorm_fp_vec_kernel(LnFpParams
         }
       }
     }
-    const float var = lf_block_sum(m2, red, tid) * inv_n;
+    const float var = lf_block_sum(m2, red, tid, red_k) * inv_n;
     const float rstd = 1.0f / sqrtf(var + p.eps);
 
 #pragma unroll
@@ -189,7 +193,8 @@ template <> __device__ __forceinline__ float lf_store1<bf16_t>(void* p, int64_t 
 // Any column count / alignment: one row per workgroup, the row is read once per pass (it stays in L2).
 template <typename T>
 __global__ __launch_bounds__(LF_THREADS) void layernorm_fp_any_kernel(LnFpParams p) {
-  __shared__ float red[LF_WAVES];
+  __shared__ float red[2 * LF_WAVES];
+  int red_k = 0;
   const int tid = threadIdx.x;
   const int row = blockIdx.x;
   const int64_t xo = (int64_t)row * p.x_rs;
@@ -198,14 +203,14 @@ __global__ __launch_bounds__(LF_THREADS) void layernorm_fp_any_kernel(LnFpParams
   if (!p.rms) {
     float s = 0.0f;
     for (int i = tid; i < p.cols; i += LF_THREADS) s += lf_load1<T>(p.x, xo + i);
-    mean = lf_block_sum(s, red, tid) * inv_n;
+    mean = lf_block_sum(s, red, tid, red_k) * inv_n;
   }
   float m2 = 0.0f;
   for (int i = tid; i < p.cols; i += LF_THREADS) {
     const float d = lf_load1<T>(p.x, xo + i) - mean;
     m2 += d * d;
   }
-  const float var = lf_block_sum(m2, red, tid) * inv_n;
+  const float var = lf_block_sum(m2, red, tid, red_k) * inv_n;
   const float rstd = 1.0f / sqrtf(var + p.eps);
   for (int i = tid; i < p.cols; i += LF_THREADS) {
     const float t = ((lf_load1<T>(p.x, xo + i) - mean) * rstd) * lf_load1<T>(p.gamma, i);

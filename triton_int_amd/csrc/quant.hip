@@ -7,6 +7,8 @@
 // reference helper's.  One workgroup walks whole rows.  Aligned rows of up to 32768 elements are
 // held in registers between the maximum and the quantisation (one read: 5 bytes of HBM traffic per
 // fp32 element, 3 per fp16 element); other rows are read twice.
+#include <type_traits>
+
 #include "ti_common.h"
 
 namespace ti {
@@ -20,13 +22,60 @@ struct QtVec<float> { typedef float type __attribute__((ext_vector_type(4))); };
 template <>
 struct QtVec<_Float16> { typedef _Float16 type __attribute__((ext_vector_type(4))); };
 
-__device__ __forceinline__ float block_max(float v, float* red, int tid) {
+// `red` holds two sets of per-wave maxima that consecutive rows (counted by `k`) alternate between, so one
+// barrier per row is enough: a wave that runs ahead writes the set the slower waves are not reading
+__device__ __forceinline__ float block_max(float v, float* red, int tid, int& k) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-  __syncthreads();  // protect `red` from the previous row
-  if ((tid & 63) == 0) red[tid >> 6] = v;
+  float* set = red + (k & 1) * (QT_THREADS / 64);
+  ++k;
+  if ((tid & 63) == 0) set[tid >> 6] = v;
   __syncthreads();
-  return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  return fmaxf(fmaxf(set[0], set[1]), fmaxf(set[2], set[3]));
+}
+
+// x / s for a whole row of x, correctly rounded like the division instruction sequence the compiler emits
+// for `x / s`, at half its cost per element.  That sequence is: scale both operands into a safe range,
+// r = refined reciprocal of the divisor (v_rcp_f32 and one Newton step: two fma), then for the dividend
+// q0 = n * r, two residual corrections (four fma, the last one carrying the range scaling back), and a
+// fix-up of the special cases.  The reciprocal part depends on the divisor only, so a row computes it once;
+// with the divisor in [2^-100, 2^100] and |n| not far above it (here |n / s| <= 127) no operand needs the
+// range scaling and no special case arises, and the five per-element operations below are the same five,
+// on the same values: the same bits.  Divisors outside that range (an all-zero row in fp16, infinities) take
+// the ordinary division.
+struct RowDivisor {
+  float s, r;
+  bool direct;
+  __device__ __forceinline__ explicit RowDivisor(float s_) : s(s_) {
+    direct = s_ >= 0x1p-100f && s_ <= 0x1p100f;
+    const float r0 = __builtin_amdgcn_rcpf(s_);
+    const float e0 = __builtin_fmaf(-s_, r0, 1.0f);
+    r = __builtin_fmaf(e0, r0, r0);
+  }
+  __device__ __forceinline__ float divide(float n) const {
+    if (!direct) return n / s;
+    const float q0 = n * r;
+    const float e1 = __builtin_fmaf(-s, q0, n);
+    const float q1 = __builtin_fmaf(e1, r, q0);
+    const float e2 = __builtin_fmaf(-s, q1, n);
+    return __builtin_fmaf(e2, r, q1);
+  }
+};
+
+// t.div_(max_val) rounded to T, round_() (half to even, exact in T), clamp_(-128, 127), to int8.  For fp16 the
+// rounding and the clamp run on the half itself (no trip back to fp32).  A NaN quotient gives -128; finite
+// rows never produce one.
+template <typename T>
+__device__ __forceinline__ int quant_one(const RowDivisor& by_scale, T v) {
+  const T d = (T)by_scale.divide((float)v);
+  if constexpr (std::is_same<T, _Float16>::value) {
+    const _Float16 r = __builtin_rintf16(d);
+    const _Float16 c = __builtin_fminf16(__builtin_fmaxf16(r, (_Float16)-128.0f), (_Float16)127.0f);
+    return (int)(short)c;
+  } else {
+    const float r = __builtin_rintf((float)d);
+    return (int)fminf(fmaxf(r, -128.0f), 127.0f);
+  }
 }
 
 template <typename T, bool VEC>
@@ -34,7 +83,8 @@ __global__ __launch_bounds__(QT_THREADS) void quant_per_token_kernel(const T* __
                                                                      int8_t* __restrict__ q, int64_t q_rs,
                                                                      T* __restrict__ scale_out, int rows, int cols) {
   typedef typename QtVec<T>::type V4;
-  __shared__ float red[QT_THREADS / 64];
+  __shared__ float red[2 * (QT_THREADS / 64)];
+  int red_k = 0;
   const int tid = threadIdx.x;
   for (int row = blockIdx.x; row < rows; row += gridDim.x) {
     const T* xr = x + (int64_t)row * x_rs;
@@ -48,17 +98,13 @@ __global__ __launch_bounds__(QT_THREADS) void quant_per_token_kernel(const T* __
     } else {
       for (int c = tid; c < cols; c += QT_THREADS) m = fmaxf(m, fabsf((float)xr[c]));
     }
-    m = block_max(m, red, tid);
+    m = block_max(m, red, tid, red_k);
     // clamp(min = 1e-8) and the division by 127, each rounded to T
     const T clamped = (T)fmaxf(m, 1e-8f);
     const T scale = (T)((float)clamped / 127.0f);
     if (tid == 0 && scale_out) scale_out[row] = scale;
-    const float s = (float)scale;
-    auto one = [&](T v) -> int {
-      const T d = (T)((float)v / s);                 // t.div_(max_val): rounded to T
-      const float r = __builtin_rintf((float)d);     // round_(): half to even, exact in T
-      return (int)fminf(fmaxf(r, -128.0f), 127.0f);  // clamp_(-128, 127); NaN -> -128 -> never produced by finite rows
-    };
+    const RowDivisor by_scale((float)scale);
+    auto one = [&](T v) -> int { return quant_one<T>(by_scale, v); };
     if constexpr (VEC) {
       for (int c = tid * 4; c < cols; c += QT_THREADS * 4) {
         const V4 v = *(const V4*)(xr + c);
@@ -77,7 +123,8 @@ __global__ __launch_bounds__(QT_THREADS) void quant_per_token_reg_kernel(const T
                                                                          int8_t* __restrict__ q, int64_t q_rs,
                                                                          T* __restrict__ scale_out, int rows, int cols) {
   typedef typename QtVec<T>::type V4;
-  __shared__ float red[QT_THREADS / 64];
+  __shared__ float red[2 * (QT_THREADS / 64)];
+  int red_k = 0;
   const int tid = threadIdx.x;
   const int nvec = cols >> 2;
   for (int row = blockIdx.x; row < rows; row += gridDim.x) {
@@ -94,16 +141,12 @@ __global__ __launch_bounds__(QT_THREADS) void quant_per_token_reg_kernel(const T
 #pragma unroll
     for (int j = 0; j < VPT; ++j)
       m = fmaxf(fmaxf(m, fabsf((float)xv[j][0])), fmaxf(fabsf((float)xv[j][1]), fmaxf(fabsf((float)xv[j][2]), fabsf((float)xv[j][3]))));
-    m = block_max(m, red, tid);
+    m = block_max(m, red, tid, red_k);
     const T clamped = (T)fmaxf(m, 1e-8f);
     const T scale = (T)((float)clamped / 127.0f);
     if (tid == 0 && scale_out) scale_out[row] = scale;
-    const float s = (float)scale;
-    auto one = [&](T v) -> int {
-      const T d = (T)((float)v / s);
-      const float r = __builtin_rintf((float)d);
-      return (int)fminf(fmaxf(r, -128.0f), 127.0f);
-    };
+    const RowDivisor by_scale((float)scale);
+    auto one = [&](T v) -> int { return quant_one<T>(by_scale, v); };
 #pragma unroll
     for (int j = 0; j < VPT; ++j) {
       const int v = tid + j * QT_THREADS;

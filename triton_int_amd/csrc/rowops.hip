@@ -23,15 +23,19 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
-// Sum over the workgroup; every thread returns the same bits (fixed combination order).
-__device__ __forceinline__ float block_sum(float v, float* red, int tid) {
+// Sum over the workgroup; every thread returns the same bits (fixed combination order).  `red` holds two
+// sets of per-wave partial sums and consecutive reductions (counted by `k`) alternate between them, so one
+// barrier per reduction is enough: a wave that runs ahead writes the set the slower waves are not reading
+// (they finished with it before the barrier in between).
+__device__ __forceinline__ float block_sum(float v, float* red, int tid, int& k) {
   v = wave_sum(v);
-  __syncthreads();  // protect `red` from the previous use
-  if ((tid & 63) == 0) red[tid >> 6] = v;
+  float* set = red + (k & 1) * RN_WAVES;
+  ++k;
+  if ((tid & 63) == 0) set[tid >> 6] = v;
   __syncthreads();
-  float s = red[0];
+  float s = set[0];
 #pragma unroll
-  for (int w = 1; w < RN_WAVES; ++w) s += red[w];
+  for (int w = 1; w < RN_WAVES; ++w) s += set[w];
   return s;
 }
 
@@ -65,7 +69,8 @@ __device__ __forceinline__ float norm_one(float x, float mean, float rstd, float
 // before the current row's reductions so that they are in flight during the two block-wide sums.
 template <int VPT, bool DQ>
 __global__ __launch_bounds__(RN_THREADS) void rownorm_vec_kernel(RowNormParams p) {
-  __shared__ float red[RN_WAVES];
+  __shared__ float red[2 * RN_WAVES];
+  int red_k = 0;
   const int tid = threadIdx.x;
   const int nvec = p.cols >> 2;
   const bool has_b = p.beta != nullptr;
@@ -133,7 +138,7 @@ __global__ __launch_bounds__(RN_THREADS) void rownorm_vec_kernel(RowNormParams p
       float s = 0.0f;
 #pragma unroll
       for (int j = 0; j < VPT; ++j) s += (x[j][0] + x[j][1]) + (x[j][2] + x[j][3]);
-      mean = block_sum(s, red, tid) * inv_n;
+      mean = block_sum(s, red, tid, red_k) * inv_n;
     }
     float m2 = 0.0f;
 #pragma unroll
@@ -144,7 +149,7 @@ __global__ __launch_bounds__(RN_THREADS) void rownorm_vec_kernel(RowNormParams p
         m2 += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
       }
     }
-    const float var = block_sum(m2, red, tid) * inv_n;
+    const float var = block_sum(m2, red, tid, red_k) * inv_n;
     const float rstd = 1.0f / sqrtf(var + p.eps);
     if (tid == 0) {
       if (p.mean_out) p.mean_out[row] = mean;
@@ -177,7 +182,8 @@ __global__ __launch_bounds__(RN_THREADS) void rownorm_vec_kernel(RowNormParams p
 // Any column count / alignment: the row is re-read from memory for each pass (it stays in L2).
 template <bool DQ>
 __global__ __launch_bounds__(RN_THREADS) void rownorm_any_kernel(RowNormParams p) {
-  __shared__ float red[RN_WAVES];
+  __shared__ float red[2 * RN_WAVES];
+  int red_k = 0;
   const int tid = threadIdx.x;
   const int row = blockIdx.x;
   const float* xr;
@@ -201,14 +207,14 @@ __global__ __launch_bounds__(RN_THREADS) void rownorm_any_kernel(RowNormParams p
   if (!p.rms) {
     float s = 0.0f;
     for (int i = tid; i < p.cols; i += RN_THREADS) s += xr[i];
-    mean = block_sum(s, red, tid) * inv_n;
+    mean = block_sum(s, red, tid, red_k) * inv_n;
   }
   float m2 = 0.0f;
   for (int i = tid; i < p.cols; i += RN_THREADS) {
     const float d = xr[i] - mean;
     m2 += d * d;
   }
-  const float var = block_sum(m2, red, tid) * inv_n;
+  const float var = block_sum(m2, red, tid, red_k) * inv_n;
   const float rstd = 1.0f / sqrtf(var + p.eps);
   if (tid == 0) {
     if (p.mean_out) p.mean_out[row] = mean;
