@@ -499,6 +499,17 @@ def decoder_layer_ms(torch, dev):
         layers[state["i"]](x)
 
     out = {"prefill_1x2048_ms": time_region(torch, prefill, 10, 2)}
+    # the same two layers replayed from a HIP graph: the nine launches of a layer back to back, without the
+    # bubbles the Python launch path leaves behind the short kernels
+    pgraph, pside = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+    with torch.cuda.stream(pside):
+        prefill(); prefill()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(pgraph, stream=pside):
+            prefill(); prefill()
+    torch.cuda.synchronize()
+    out["prefill_1x2048_graph_ms"] = time_region(torch, pgraph.replay, 10, 2) / 2
+    del pgraph
     # per-stage breakdown of the prefill, in sequence: stream events between the stages of the same
     # alternating forward passes (weights cold, clocks as the whole layer holds them)
     reps, marks = 8, []
