@@ -367,6 +367,19 @@ def extras(torch, dev):
                                    "grouped_launch_ms": tg, "grouped_launch_TOPS": ops3 / tg / 1e9,
                                    "three_launches_ms_rounds": t3s, "grouped_launch_ms_rounds": tgs}
     del xq, w3, b3, o3, outs
+    # the control for "what bounds a short launch": the 2048 x 4096 x 4096 int8 GEMM of the linear set on uniform
+    # random and on all-zero operands (same instructions, same bytes, less switching), back to back
+    xu, wu = torch.randint(-127, 128, (2048, 4096), dtype=torch.int8, device=dev), torch.randint(-127, 128, (4096, 4096), dtype=torch.int8, device=dev)
+    xz, wz = torch.zeros_like(xu), torch.zeros_like(wu)
+    bq = torch.randint(-127, 128, (4096,), dtype=torch.int8, device=dev)
+    alq, beq, oq = torch.tensor(0.002, device=dev), torch.tensor(0.01, device=dev), torch.empty((2048, 4096), dtype=torch.int8, device=dev)
+    rec = {}
+    for rnd in range(3):
+        for name, (xx, ww) in (("uniform", (xu, wu)), ("zeros", (xz, wz))):
+            rec.setdefault(name, []).append(time_region(torch, lambda: linear.linear_a8_w8_b8_o8(xx, ww, bq, alq, beq, out=oq), 50, 5))
+    out["gemm_2048x4096x4096_uniform_vs_zero_operands"] = {
+        k: {"us": sorted(v)[1] * 1e3, "TOPS": 2.0 * 2048 * 4096 * 4096 / sorted(v)[1] / 1e9} for k, v in rec.items()}
+    del xu, wu, xz, wz, oq
     # a yardstick, not part of the path: the vendor library's int8 GEMM (torch._int_mm, int32 out) on
     # the fc1 shape with the same kind of operands, next to this library's int32-output linear
     try:

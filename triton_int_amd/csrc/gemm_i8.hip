@@ -24,6 +24,15 @@
 
 namespace ti {
 
+#ifdef TI_GEMM_TIMELINE
+// experiment builds only: per workgroup, the constant-rate clock (100 MHz) at a few points of the
+// wave-specialised kernel, read back by ti_debug_timeline
+__device__ unsigned long long g_timeline[1024 * 8];
+#define TI_TL(slot) do { if ((threadIdx.x & 63) == 0) g_timeline[blockIdx.x * 8 + (slot)] = wall_clock64(); } while (0)
+#else
+#define TI_TL(slot) do { } while (0)
+#endif
+
 struct GemmParams {
   const int8_t* A;
   const int8_t* B;
@@ -1429,10 +1438,12 @@ __global__ __launch_bounds__((WAVES_M * WAVES_N + PW) * 64) void gemm_mfma_ws_ke
         aim(i_issue);
       }
     };
+    if (wave == NWC) TI_TL(0);
     aim(0);
 #pragma unroll
     for (int t = 0; t < DEPTH; ++t) issue_ktile();
     wait_loads_and_barrier<LOADS*(DEPTH - 1)>();  // k-tile 0 landed
+    if (wave == NWC) TI_TL(1);
     int total = count * KT;  // k-tiles of all items = barriers to join
     if (SPL > 1) {
       total = 0;
@@ -1580,9 +1591,12 @@ __global__ __launch_bounds__((WAVES_M * WAVES_N + PW) * 64) void gemm_mfma_ws_ke
       }
       if (lane == 0) atomicExch(p.sk_counter + rank * NWC + wave, 0);
     }
+    if (wave == 0 && it == 0) TI_TL(2);
     stream_epilogue<TM, TN, OUTCLS>(p, e, acc, bz, m0 + wm * WTM, n0 + wn * WTN,
                                     lds + NSTAGE * STAGE + wave * (STRIP + COLS), lane);
+    if (wave == 0 && it == 0) TI_TL(3);
   }
+  if (wave == 0) TI_TL(4);
 }
 
 // ---- gather family -----------------------------------------------------------------------------
@@ -2877,6 +2891,12 @@ int ti_gemm_plan(const int8_t* A, int64_t sAb, int64_t sAm, int64_t sAk, const i
 int ti_release_workspaces(void* stream, int all_streams, int64_t* freed_bytes) {
   return ti::sk_release((hipStream_t)stream, all_streams != 0, freed_bytes);
 }
+
+#ifdef TI_GEMM_TIMELINE
+int ti_debug_timeline(unsigned long long* host, int n) {
+  return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(ti::g_timeline), sizeof(unsigned long long) * n);
+}
+#endif
 
 int ti_gemm_num_configs(void) { return ti::g_num_configs; }
 
