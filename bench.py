@@ -450,7 +450,8 @@ def m_sweep(torch, dev, N, K, lib, full=True):
 
 def cpu_baseline_rows(torch, budget_s=4.0):
     """CPU emulation (torch on the host cores) of the HBM-bound kernels on bounded samples of their
-    benchmark shapes: dq + add + LayerNormQ (functional/fused.py:6-15), GELU-quant, one head of Q.K^T."""
+    benchmark shapes: dq + add + LayerNormQ (functional/fused.py:6-15), GELU-quant, one head of Q.K^T,
+    and of the single 512 x 768 x 768 int8 linear."""
     import torch.nn.functional as F
 
     from oracle import cpu_emulation as E
@@ -481,6 +482,12 @@ def cpu_baseline_rows(torch, budget_s=4.0):
     r = timed(lambda: E.bmm_o8(q, k, 1e-3), 512 * 128 + 2048 * 128 + 512 * 2048, "512 query rows of one of 160 heads, 2048 keys")
     r["TOPS"] = 2.0 * 512 * 2048 * 128 / (r["ms"] * 1e-3) / 1e12
     out["bmm_qk_s8"] = r
+    x1 = torch.randint(-127, 128, (512, 768), dtype=torch.int8, generator=g)
+    w1 = torch.randint(-127, 128, (768, 768), dtype=torch.int8, generator=g)
+    b1 = torch.randint(-127, 128, (768,), dtype=torch.int8, generator=g)
+    r = timed(lambda: E.linear_o8(x1, w1, b1, 0.0021, 0.013), 512 * 768 * 2 + 768 * 768 + 768, "the whole 512 x 768 x 768 linear")
+    r["TOPS"] = 2.0 * 512 * 768 * 768 / (r["ms"] * 1e-3) / 1e12
+    out["single_linear_512x768x768"] = r
     return out
 
 
