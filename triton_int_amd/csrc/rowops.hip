@@ -67,6 +67,23 @@ __device__ __forceinline__ float norm_one(float x, float mean, float rstd, float
 // row-invariant and stay in registers for all of them (re-reading them per row would triple the
 // bytes that cross the L2 -> CU path), and for the plain LayerNorm the next row's loads are issued
 // before the current row's reductions so that they are in flight during the two block-wide sums.
+//
+// Every access to a row goes through a buffer descriptor of that row (range-checked: vectors past the
+// row's end load zeros and store nothing), so the loop has no branch around a memory instruction.  That
+// matters for more than the branches: with straight-line code the compiler can count the memory
+// operations between a load and its use, and the wait at the top of an iteration becomes "all but the
+// stores issued since" instead of "everything", i.e. the next row's reductions no longer wait for the
+// previous row's stores to be acknowledged by the L2.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t row_rsrc(const void* row_ptr, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc((void*)row_ptr, 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ v4f row_load_f4(__amdgpu_buffer_rsrc_t r, int vec) {
+  return __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, vec * 16, 0, 2));  // 2: non-temporal
+}
+__device__ __forceinline__ void row_store_f4(__amdgpu_buffer_rsrc_t r, int vec, v4f v) {
+  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, v), r, vec * 16, 0, 2);
+}
+
 template <int VPT, bool DQ>
 __global__ __launch_bounds__(RN_THREADS) void rownorm_vec_kernel(RowNormParams p) {
   __shared__ float red[2 * RN_WAVES];
@@ -75,29 +92,29 @@ __global__ __launch_bounds__(RN_THREADS) void rownorm_vec_kernel(RowNormParams p
   const int nvec = p.cols >> 2;
   const bool has_b = p.beta != nullptr;
   const v4f zero4 = {0.f, 0.f, 0.f, 0.f};
+  const unsigned row_bytes = (unsigned)p.cols * 4u;
 
   v4f w[VPT], b[VPT];
-#pragma unroll
-  for (int j = 0; j < VPT; ++j) {
-    const int v = tid + j * RN_THREADS;
-    w[j] = v < nvec ? *(const v4f*)(p.gamma + v * 4) : zero4;
-    b[j] = (has_b && v < nvec) ? *(const v4f*)(p.beta + v * 4) : zero4;
-  }
-
-  auto load_x = [&](int row, v4f (&dst)[VPT]) {
+  {
+    const __amdgpu_buffer_rsrc_t rg = row_rsrc(p.gamma, row_bytes), rb = row_rsrc(p.beta, has_b ? row_bytes : 0u);
 #pragma unroll
     for (int j = 0; j < VPT; ++j) {
-      const int v = tid + j * RN_THREADS;
-      // streamed once: non-temporal
-      dst[j] = v < nvec ? __builtin_nontemporal_load((const v4f*)(p.x + (int64_t)row * p.x_rs + v * 4)) : zero4;
+      w[j] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rg, (tid + j * RN_THREADS) * 16, 0, 0));
+      b[j] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rb, (tid + j * RN_THREADS) * 16, 0, 0));
     }
+  }
+
+  // a row at or past p.rows gets an empty descriptor: its loads touch no memory
+  auto load_x = [&](int row, v4f (&dst)[VPT]) {
+    const bool in = row < p.rows;
+    const __amdgpu_buffer_rsrc_t rx = row_rsrc(p.x + (int64_t)(in ? row : 0) * p.x_rs, in ? row_bytes : 0u);
+#pragma unroll
+    for (int j = 0; j < VPT; ++j) dst[j] = row_load_f4(rx, tid + j * RN_THREADS);
   };
 
   v4f x[VPT], xn[VPT];
   int row = blockIdx.x;
-  if constexpr (!DQ) {
-    if (row < p.rows) load_x(row, xn);
-  }
+  if constexpr (!DQ) load_x(row, xn);
   const float inv_n = 1.0f / (float)p.cols;
   const bool y_vec = p.y && ((p.y_rs & 3) == 0) && ((((uintptr_t)p.y) & 3) == 0);
   float in_scale = p.in_scale;
@@ -107,30 +124,32 @@ __global__ __launch_bounds__(RN_THREADS) void rownorm_vec_kernel(RowNormParams p
 
   for (; row < p.rows; row += gridDim.x) {
     if constexpr (DQ) {
+      const __amdgpu_buffer_rsrc_t ra = row_rsrc(p.acc + (int64_t)row * p.acc_rs, row_bytes);
+      const __amdgpu_buffer_rsrc_t rr = row_rsrc(p.resid_in + (int64_t)row * p.rin_rs, row_bytes);
+      const __amdgpu_buffer_rsrc_t ro = row_rsrc(p.resid_out + (int64_t)row * p.rout_rs, row_bytes);
+      v4i a[VPT];
+      v4f r[VPT];
 #pragma unroll
       for (int j = 0; j < VPT; ++j) {
-        const int v = tid + j * RN_THREADS;
-        if (v < nvec) {
-          const v4i a = __builtin_nontemporal_load((const v4i*)(p.acc + (int64_t)row * p.acc_rs + v * 4));
-          const v4f r = __builtin_nontemporal_load((const v4f*)(p.resid_in + (int64_t)row * p.rin_rs + v * 4));
-          v4f o;
+        a[j] = __builtin_amdgcn_raw_buffer_load_b128(ra, (tid + j * RN_THREADS) * 16, 0, 2);
+        r[j] = row_load_f4(rr, tid + j * RN_THREADS);
+      }
 #pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            // functional/fused.py:9: residual + alpha * int32 (product and sum rounded separately)
-            const float prod = in_scale * (float)a[t];
-            o[t] = r[t] + prod;
-          }
-          x[j] = o;
-          __builtin_nontemporal_store(o, (v4f*)(p.resid_out + (int64_t)row * p.rout_rs + v * 4));
-        } else {
-          x[j] = zero4;
+      for (int j = 0; j < VPT; ++j) {
+        v4f o;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          // functional/fused.py:9: residual + alpha * int32 (product and sum rounded separately)
+          const float prod = in_scale * (float)a[j][t];
+          o[t] = r[j][t] + prod;
         }
+        x[j] = o;  // vectors past the row's end: 0 + scale * 0
+        row_store_f4(ro, tid + j * RN_THREADS, o);
       }
     } else {
 #pragma unroll
       for (int j = 0; j < VPT; ++j) x[j] = xn[j];
-      const int next = row + (int)gridDim.x;
-      if (next < p.rows) load_x(next, xn);
+      load_x(row + (int)gridDim.x, xn);
     }
 
     float mean = 0.0f;
@@ -156,24 +175,21 @@ __global__ __launch_bounds__(RN_THREADS) void rownorm_vec_kernel(RowNormParams p
       if (p.rstd_out) p.rstd_out[row] = rstd;
     }
 
+    const __amdgpu_buffer_rsrc_t rl = row_rsrc(p.ln_out ? p.ln_out + (int64_t)row * p.ln_rs : nullptr, p.ln_out ? row_bytes : 0u);
+    const __amdgpu_buffer_rsrc_t ry = row_rsrc(p.y ? p.y + (int64_t)row * p.y_rs : nullptr, y_vec ? (unsigned)p.cols : 0u);
 #pragma unroll
     for (int j = 0; j < VPT; ++j) {
       const int v = tid + j * RN_THREADS;
-      if (v < nvec) {
-        v4f o;
+      v4f o;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) o[t] = norm_one(x[j][t], mean, rstd, w[j][t], b[j][t], has_b);
-        if (p.ln_out) __builtin_nontemporal_store(o, (v4f*)(p.ln_out + (int64_t)row * p.ln_rs + v * 4));
-        if (p.y) {
-          const int q0 = q8(o[0], p.round_mode), q1 = q8(o[1], p.round_mode), q2 = q8(o[2], p.round_mode),
-                    q3 = q8(o[3], p.round_mode);
-          int8_t* dst = p.y + (int64_t)row * p.y_rs + v * 4;
-          if (y_vec) {
-            __builtin_nontemporal_store(pack4(q0, q1, q2, q3), (unsigned*)dst);
-          } else {
-            dst[0] = (int8_t)q0; dst[1] = (int8_t)q1; dst[2] = (int8_t)q2; dst[3] = (int8_t)q3;
-          }
-        }
+      for (int t = 0; t < 4; ++t) o[t] = norm_one(x[j][t], mean, rstd, w[j][t], b[j][t], has_b);
+      row_store_f4(rl, v, o);  // an empty descriptor when there is no fp32 output
+      const int q0 = q8(o[0], p.round_mode), q1 = q8(o[1], p.round_mode), q2 = q8(o[2], p.round_mode),
+                q3 = q8(o[3], p.round_mode);
+      __builtin_amdgcn_raw_buffer_store_b32((int)pack4(q0, q1, q2, q3), ry, v * 4, 0, 2);
+      if (p.y && !y_vec && v < nvec) {  // int8 rows that are not 4-byte aligned
+        int8_t* dst = p.y + (int64_t)row * p.y_rs + v * 4;
+        dst[0] = (int8_t)q0; dst[1] = (int8_t)q1; dst[2] = (int8_t)q2; dst[3] = (int8_t)q3;
       }
     }
   }
@@ -247,11 +263,17 @@ static int launch_rownorm(const RowNormParams& p, hipStream_t stream) {
     return launch_status("rownorm_any_kernel");
   }
   const int vpt = (p.cols / 4 + RN_THREADS - 1) / RN_THREADS;
-  // persistent workgroups: a few per CU, each walking several rows.  Measured at 8192 rows: plain
-  // LayerNormQ of 5120 columns 40.2 us with 4 per CU, 37.5 us with 3, 39.3 us with 2 (4096 columns:
-  // 31.1 / 31.5 / 34.7 us); the dq + add variant 95 / 102 / 129 us.  Two rows ahead instead of one
-  // in flight per workgroup: 46 us.
-  const unsigned slots = 256u * (vpt <= 2 ? 8u : (vpt <= 4 ? 4u : (vpt == 5 ? (DQ ? 4u : 3u) : 3u)));
+  // persistent workgroups: a few per CU, each walking several rows.  Measured at 8192 rows with 2 / 3 / 4 / 8
+  // workgroups per CU (us): plain LayerNormQ of 5120 columns 36.5 / 37.6 / 39.1 / -, of 4096 columns
+  // 32.1 / 30.6 / 31.6 / -, of 3072 columns 28.1 / 24.7 / 24.8 / 26.3, of 2048 columns 23.8 / 19.8 / 19.1 / 17.9,
+  // of 8192 columns 58.1 / 67.6 / 61.5 / 65.9; the dq + add variant of 5120 columns 90.4 / 96.4 / 97.4 / -, of
+  // 4096 columns 73.1 / 73.9 / 74.9 / -, of 2048 columns 42.4 / 36.4 / 38.8 / 40.5.  (16384 rows rank the same.)
+  // Plain LayerNormQ of 5120 columns with 2 per CU is the fastest in a quiet machine (and by 9-13 % from 16384 rows
+  // on) but the most exposed to the slower memory phases the chip goes through in its first few hundred launches
+  // (36-45 us at 8192 rows where 3 per CU stay at 37-40), so it takes 2 only where the margin is large.
+  const unsigned ln_per_cu = vpt <= 2 ? 8u : (vpt == 3 ? 4u : (vpt >= 6 || (vpt == 5 && p.rows >= 16384) ? 2u : 3u));
+  const unsigned per_cu = DQ ? (vpt <= 2 ? 3u : 2u) : ln_per_cu;
+  const unsigned slots = 256u * per_cu;
   if (grid.x > slots) grid.x = slots;
   if (vpt <= 1) rownorm_vec_kernel<1, DQ><<<grid, block, 0, stream>>>(p);
   else if (vpt <= 2) rownorm_vec_kernel<2, DQ><<<grid, block, 0, stream>>>(p);
