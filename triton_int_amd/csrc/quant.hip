@@ -4,7 +4,7 @@
 // for fp32 and fp16 activations.  Every step is rounded to the tensor's dtype as torch's elementwise
 // kernels do (fp16: computed in fp32, rounded to fp16 after the clamp, after the division by 127 and
 // after the division of each element), so the int8 result and the scale are bit-identical to the
-// reference helper's.  One workgroup walks whole rows.  Aligned rows of up to 32768 elements are
+// reference helper's.  One workgroup per row.  Aligned rows of up to 32768 elements are
 // held in registers between the maximum and the quantisation (one read: 5 bytes of HBM traffic per
 // fp32 element, 3 per fp16 element); other rows are read twice.
 #include <type_traits>

@@ -6,7 +6,7 @@
 // zhanglei1172/triton_int), supplies the native dq_add_layernorm_q the reference only emulates
 // (functional/fused.py:6-32) and a launchable form of fast_geluQ (kernels/fused.py:76-79).
 //
-// Row kernels: one row per 256-thread workgroup.  The whole row sits in registers as float4
+// Row kernels: a 256-thread workgroup per row at a time.  The whole row sits in registers as float4
 // vectors (thread t owns vectors t, t+256, ...: every load/store instruction of a wave is one
 // contiguous 1 KB / 256 B run), so x is read from HBM exactly once; mean and the centred sum of
 // squares are exact two-pass statistics reduced with wave shuffles and one LDS hop.
