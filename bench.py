@@ -9,6 +9,10 @@ hidden 4096): q/k/v/out W8A8B8O8 4096x4096, fc1 4096->16384 with the GELU-quant 
 Prints ONE JSON line: whole-step int8 TOPS, the roofline of the dominant GEMM kernel (timed with
 events on the launch stream), the CPU emulation baseline on a bounded row sample, and — under
 "extra" — GB/s of the row kernels and the attention BMMs.
+
+Set-up (untimed, before the W warm-up steps) runs the step for --settle-ms (default 40 ms) and reports what
+those steps took under "cold_start": the first ~15 ms of heavy work of a process are a transient of the
+chip's power management (a few steps at the boost clock, then ~25 steps well below the level it settles on).
 """
 from __future__ import annotations
 
@@ -601,6 +605,11 @@ def main():
     ap.add_argument("--rownorm-only", action="store_true",
                     help="run 6 launches of LayerNormQ and 3 of dq + add + LayerNormQ on 8192 x 5120 and exit: the "
                          "program profiled for the row-norm counter summary")
+    ap.add_argument("--settle-ms", type=float, default=40.0,
+                    help="during set-up, before the warm-up steps, run untimed steps for this long (each one timed "
+                         "on its own and reported under \"cold_start\"): the first ~15 ms of heavy work after a "
+                         "process starts are a transient of the chip's power management (three steps at the boost "
+                         "clock, then ~25 steps 10-25 %% slower than the level it settles on); 0 turns it off")
     ap.add_argument("--calib-copy-mb", type=int, default=0,
                     help="before the timed region, run 4 device-to-device copies of this many MiB: a kernel of "
                          "known traffic to scale rocprofv3's FETCH_SIZE / WRITE_SIZE readings with")
@@ -756,35 +765,57 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    # Settling (set-up, untimed): what a step costs in the first milliseconds of heavy work of a process is a
+    # property of the chip's power management, not of the kernels, and is reported separately.
+    cold = None
+    sclk_samples = []
+    if args.settle_ms > 0:
+        # the shader clock the chip holds under the steps: the driver's sysfs file read from a thread, here and
+        # not in the timed region (2 000 reads a second cost the timed steps 4-5 %)
+        import glob
+        import threading
+
+        sclk_file, sampling = _find_sclk_file(torch, glob), {"on": True}
+
+        def sample_sclk():
+            time.sleep(0.02)  # past the transient
+            while sampling["on"] and len(sclk_samples) < 400:
+                mhz = _read_sclk_mhz(sclk_file)
+                if mhz:
+                    sclk_samples.append(mhz)
+                time.sleep(0.001)
+
+        th = threading.Thread(target=sample_sclk)
+        if sclk_file:
+            th.start()
+        marks = [torch.cuda.Event(enable_timing=True) for _ in range(401)]
+        n_settle, t_s = 0, time.perf_counter()
+        marks[0].record()
+        while n_settle < 400 and (time.perf_counter() - t_s) * 1e3 < args.settle_ms:
+            for _ in range(10):  # launches are asynchronous: wait per block so that the limit is device time
+                step()
+                n_settle += 1
+                marks[n_settle].record()
+            torch.cuda.synchronize()
+        sampling["on"] = False
+        if sclk_file:
+            th.join()
+        ts = [marks[i].elapsed_time(marks[i + 1]) for i in range(n_settle)]
+        blocks = [ts[i:i + 5] for i in range(0, len(ts), 5)]
+        cold = {"steps": n_settle,
+                "tops_per_block_of_5_steps": [round(total_ops / (sum(b) / len(b) * 1e-3) / 1e12) for b in blocks],
+                "note": "untimed set-up steps before the warm-up, from the first heavy launches of the process on "
+                        "(device time per block of 5 steps): boost clock, then the power management's "
+                        "over-correction, then the level the timed steps run at"}
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
     events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-    # the shader clock the chip holds during the timed steps: the driver's sysfs file read from a thread
-    # (in-process, no child; the region is short, so the thread reads back to back)
-    import glob
-    import threading
-
-    sclk_file, sclk_samples, sampling = _find_sclk_file(torch, glob), [], {"on": True}
-
-    def sample_sclk():
-        while sampling["on"] and len(sclk_samples) < 400:
-            mhz = _read_sclk_mhz(sclk_file)
-            if mhz:
-                sclk_samples.append(mhz)
-            time.sleep(0.0005)
-
-    th = threading.Thread(target=sample_sclk)
-    if sclk_file:
-        th.start()
     t0 = time.perf_counter()
     for i in range(args.steps):
         step(events[i])
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    sampling["on"] = False
-    if sclk_file:
-        th.join()
     ms_per_step = wall * 1e3 / args.steps
     dom_ms = sum(a.elapsed_time(b) for a, b in events) / args.steps  # per step, all launches of the dominant kernel
     # device time of whole steps: start event of step i to start event of step i+1
@@ -829,7 +860,7 @@ def main():
                                      for _, m, x, _ in groups[dominant]) / n_dom,
             "launches_per_step": n_dom,
             "avg_launch_us": dom_ms * 1e3 / n_dom,
-            "sclk_mhz_during_timed_steps": (sorted(sclk_samples)[len(sclk_samples) // 2] if sclk_samples else None),
+            "sclk_mhz_during_settling_steps": (sorted(sclk_samples)[len(sclk_samples) // 2] if sclk_samples else None),
             "ops_per_launch": dom_ops / n_dom,
         },
     }
@@ -838,6 +869,8 @@ def main():
     result["roofline"]["measured_mfma_issue_peak_random_operands"] = peak_rand
     result["roofline"]["measured_mfma_issue_peak_constant_operands"] = peak_const
     result["roofline"]["frac_of_measured_issue_peak"] = achieved / peak_rand
+    if cold is not None:
+        result["cold_start"] = cold
     if not args.no_extra:
         result["extra"] = extras(torch, dev)
         result["extra"]["attention_i8_fused_vs_chain_40x2048x2048"] = attention_mismatch(torch, dev)
