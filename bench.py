@@ -124,10 +124,20 @@ def cpu_baseline(torch, layers, budget_s=12.0):
     }
 
 
+SETTLE_MS = 25.0  # every timed region is preceded by this much of the same work (see "cold_start" in main)
+
+
 def time_region(torch, fn, iters, warm):
     for _ in range(warm):
         fn()
     torch.cuda.synchronize()
+    # a burst of work that follows a lighter phase starts with a transient of the chip's power management (some
+    # 15 ms: boost, over-correction, then the level it holds); the timed iterations come after it
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < SETTLE_MS:
+        for _ in range(max(1, warm)):
+            fn()
+        torch.cuda.synchronize()
     s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     s.record()
     for _ in range(iters):
