@@ -431,8 +431,12 @@ def m_sweep(torch, dev, N, K, lib, full=True):
     ms_list = (32, 64, 128, 256) + tuple(1024 * i for i in range(1, 17)) if full else (32, 64, 128, 256, 1024, 2048, 4096, 8192, 16384)
 
     def timed(a, w, bias):
-        for _ in range(3):
-            linear.linear_a8_w8_bfp32_ofp32(a, w, bias, one, one)
+        # warm-up by time, 25 ms, as the reference's do_bench does (its default), then 20 timed launches
+        t0 = time.perf_counter()
+        while (time.perf_counter() - t0) * 1e3 < SETTLE_MS:
+            for _ in range(3):
+                linear.linear_a8_w8_bfp32_ofp32(a, w, bias, one, one)
+            torch.cuda.synchronize()
         reps = 20
         ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
         for s_, e_ in ev:
