@@ -264,14 +264,14 @@ static int launch_rownorm(const RowNormParams& p, hipStream_t stream) {
   }
   const int vpt = (p.cols / 4 + RN_THREADS - 1) / RN_THREADS;
   // persistent workgroups: a few per CU, each walking several rows.  Measured at 8192 rows with 2 / 3 / 4 / 8
-  // workgroups per CU (us): plain LayerNormQ of 5120 columns 36.5 / 37.6 / 39.1 / -, of 4096 columns
-  // 32.1 / 30.6 / 31.6 / -, of 3072 columns 28.1 / 24.7 / 24.8 / 26.3, of 2048 columns 23.8 / 19.8 / 19.1 / 17.9,
-  // of 8192 columns 58.1 / 67.6 / 61.5 / 65.9; the dq + add variant of 5120 columns 90.4 / 96.4 / 97.4 / -, of
-  // 4096 columns 73.1 / 73.9 / 74.9 / -, of 2048 columns 42.4 / 36.4 / 38.8 / 40.5.  (16384 rows rank the same.)
-  // Plain LayerNormQ of 5120 columns with 2 per CU is the fastest in a quiet machine (and by 9-13 % from 16384 rows
-  // on) but the most exposed to the slower memory phases the chip goes through in its first few hundred launches
-  // (36-45 us at 8192 rows where 3 per CU stay at 37-40), so it takes 2 only where the margin is large.
-  const unsigned ln_per_cu = vpt <= 2 ? 8u : (vpt == 3 ? 4u : (vpt >= 6 || (vpt == 5 && p.rows >= 16384) ? 2u : 3u));
+  // workgroups per CU, each figure after 20 ms of the same launches (us): plain LayerNormQ of 5120 columns
+  // 35.7 / 37.5 / 39.0 / 38.6, of 4096 columns 30.9 / 30.6 / 31.1 / 31.0, of 3072 columns 27.3 / 24.2 / 24.1 / 25.3,
+  // of 2048 columns 22.8 / 18.8 / 17.8 / 17.5 (16384 rows: 41.7 / 34.1 / 31.0 / 33.7), of 8192 columns
+  // 57.1 / 63.7 / 59.0 / 62.3; the dq + add variant of 5120 columns 89.8 / 95.8 / 96.5 / 95.4, of 4096 columns
+  // 71.2 / 73.8 / 74.8 / 73.7, of 3072 columns 54.5 / 55.5 / 57.4 / 57.9, of 2048 columns 41.4 / 36.4 / 38.2 / 39.8.
+  // (In the first milliseconds of a burst, while the chip's power management settles, 2 per CU is the variant
+  // that suffers most: 36-45 us for the first of these where 3 per CU stay at 37-40.)
+  const unsigned ln_per_cu = vpt <= 2 ? 4u : (vpt <= 4 ? 3u : 2u);
   const unsigned per_cu = DQ ? (vpt <= 2 ? 3u : 2u) : ln_per_cu;
   const unsigned slots = 256u * per_cu;
   if (grid.x > slots) grid.x = slots;
