@@ -242,8 +242,11 @@ static int launch_layernorm_fp(const LnFpParams& p, hipStream_t stream) {
   // columns with 4 / 3 / 2 of them: the skip variants (two or three streams per row) run best with 2
   // (fp16 122 / 114 / 113 us, bf16 122 / 117 / 110, fp32 244 / 246 / 232), plain fp32 with 3 at 5120
   // columns (118 / 113 / 113) and 2 at 4096 (94 / 93 / 88), plain 16-bit with 4 (56 / 60 / 80)
+  // Two vectors per thread (16-bit rows of 2049 .. 4096 columns), 16384 x 4096 fp16 after 20 ms of the same
+  // launches, 8 / 6 / 4 / 3 / 2 per CU: plain 49.5 / 45.8 / 45.3 / 48.6 / 67.5 us, skip with both outputs
+  // 96.4 / 95.6 / 96.3 / 87.7 / 86.8 us.
   const unsigned mid = p.skip ? 2u : (sizeof(T) == 4 ? (vpt >= 5 ? 3u : 2u) : 4u);
-  const unsigned slots = 256u * (vpt <= 2 ? 8u : (vpt <= 5 ? mid : 2u));
+  const unsigned slots = 256u * (vpt <= 1 ? 8u : (vpt == 2 ? (p.skip ? 2u : 4u) : (vpt <= 5 ? mid : 2u)));
   const dim3 grid((unsigned)p.rows < slots ? (unsigned)p.rows : slots), block(LF_THREADS);
 #define TI_LF_LAUNCH(V) layernorm_fp_vec_kernel<T, V><<<grid, block, 0, stream>>>(p)
   if (vpt <= 1) TI_LF_LAUNCH(1);
