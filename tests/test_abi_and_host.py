@@ -216,3 +216,24 @@ def test_c_abi_status_codes_with_raw_ctypes():
     assert lib.ti_attention_i8(P, 2048, 128, P, 2048, 128, P, 2048, 16, P, 2048, 128, 1, 16, 16, 128, 1e-3, 0.0, 0.01, 0, None) == TI_E_COMBO
     assert lib.ti_qkv_decode_i8(P, 64, P, 64, 0, P, P, P, 64, 32, 64, 2048, P, 64, P, 64, 16, None) == TI_E_COMBO  # M > 16
     assert lib.ti_mfma_i8_probe(-1, 0, None, None) == TI_E_SHAPE
+
+
+def test_bench_reads_the_traffic_figure_from_the_committed_profile():
+    """bench.py's roofline.traffic is parsed out of the counters summary it names: the row and the two scale
+    factors must be there, and the figure must be what they multiply out to."""
+    import bench
+
+    kernel = "ws_256x128x128_w2x2_s1_p3_l4/int8"
+    total, source = bench.traffic_from_profile(kernel)
+    assert total is not None and source.startswith(bench.TRAFFIC_PROFILE[kernel][0])
+    assert 2.0 * 48.65e6 < total < 3.0 * 48.65e6  # 2.5x the algorithmic bytes of an average launch of the step
+    assert bench.traffic_from_profile("no such kernel") == (None, None)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "one GPU" in r.stderr
