@@ -306,7 +306,8 @@ int ti_transpose_i8(const int8_t* src, int64_t src_row_stride, int8_t* dst, int6
  *     C[m][n] = (alpha * f(acc[m][n]) + beta * bias[n]) + residual[m][n]        fp32, rounded per step
  * A [M,K], W [N,K] int8 with unit column stride, bias fp32 [N] or NULL, residual and C fp32 with unit
  * column stride (row strides in elements).  With M <= 16 the weight-streaming decode kernel adds the
- * residual as it stores (one launch instead of two); otherwise the GEMM is followed by an add kernel.
+ * residual as it stores, and the persistent kernels that serve large outputs add it in their epilogue (one
+ * launch instead of two); otherwise the GEMM is followed by an add kernel.
  * Same bits as the linear followed by an fp32 add.  C must not overlap the residual.
  */
 int ti_linear_i8_residual_f32(const int8_t* A, int64_t lda, const int8_t* W, int64_t ldw, const float* bias,

@@ -691,10 +691,12 @@ def test_decode_kernel_several_passes_strided_and_16bit_outputs():
         assert np.array_equal(got16, O.linear_a8_w8_bfp32_ofp32(a, w, bf, alpha, 1.0, out_dtype=odt))
 
 
-@pytest.mark.parametrize("M,N,K", [(16, 5120, 20480), (1, 272, 1040), (7, 5124, 1024), (300, 320, 256), (2048, 768, 512), (16, 50272, 1024)])
+@pytest.mark.parametrize("M,N,K", [(16, 5120, 20480), (1, 272, 1040), (7, 5124, 1024), (300, 320, 256), (2048, 768, 512), (16, 50272, 1024),
+                                   (2048, 5120, 1024), (1000, 4096, 512), (2049, 4100, 256), (513, 640, 128), (4096, 6848, 512)])
 def test_linear_with_residual_equals_linear_then_add(M, N, K):
-    """ti_linear_i8_residual_f32: the decode kernel's fused add (M <= 16) and the GEMM + add-kernel pair
-    give the bits of the fp32 linear followed by an fp32 add."""
+    """ti_linear_i8_residual_f32: the decode kernel's fused add (M <= 16), the persistent kernels' fused add (large
+    outputs, whole and ragged tiles) and the GEMM + add-kernel pair give the bits of the fp32 linear followed by an
+    fp32 add."""
     linear, _, _ = _kl()
     g = rng(M + N + K)
     a, w = rand_i8(g, M, K), rand_i8(g, N, K)

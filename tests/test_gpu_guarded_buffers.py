@@ -248,3 +248,30 @@ def test_gemm_stays_inside_its_views(M, N, K, batch, odt):
     acc = torch.bmm(a.view(batch, M, K).double(), b.view(batch, N, K).double().transpose(1, 2)) if M * N * K * batch < 2e9 else None
     if acc is not None and odt == torch.int32:
         assert torch.equal(hc.view.view(batch, M, N).cpu().double(), acc)
+
+
+@pytest.mark.parametrize("M,N,K", [(2048, 5120, 512), (1000, 4100, 256), (16, 5120, 2048), (300, 320, 256), (2049, 640, 128)])
+def test_linear_with_residual_stays_inside_its_views(M, N, K):
+    """ti_linear_i8_residual_f32 with the residual and the output at a pitch inside patterned / poisoned buffers
+    (the persistent kernels fetch the residual in their epilogue): equal to the same call on contiguous
+    operands, nothing written outside the output's rows."""
+    L = _lib()
+    g = rng(M * 61 + N + K)
+    a, w = _i8(g, M, K), _i8(g, N, K)
+    bias, res = _f32(g, 1, N), _f32(g, M, N) * 3
+    ha, hw = Held(M, K, torch.int8, K + 16, IN_FILL, 0, a), Held(N, K, torch.int8, K + 32, IN_FILL, 0, w)
+    hb, hr = Held(1, N, torch.float32, None, IN_FILL, 0, bias), Held(M, N, torch.float32, N + 12, IN_FILL, 0, res)
+    hc, hw2 = Held(M, N, torch.float32, N + 4, OUT_FILL), Held(M, N, torch.float32, N, OUT_FILL)
+    alpha, beta = torch.tensor([3e-4], device=DEV), torch.tensor([1.0], device=DEV)
+    print(f"ti_linear_i8_residual_f32 M={M} N={N} K={K} pitched", flush=True)
+    _ok(L.lib().ti_linear_i8_residual_f32(ha.ptr, ha.pitch, hw.ptr, hw.pitch, hb.ptr, alpha.data_ptr(), beta.data_ptr(), hr.ptr, hr.pitch,
+                                          hc.ptr, hc.pitch, M, N, K, _stream()), "ti_linear_i8_residual_f32")
+    ca, cw, cb, cr = a.to(DEV), w.to(DEV), bias.to(DEV), res.to(DEV)
+    print(f"ti_linear_i8_residual_f32 M={M} N={N} K={K} contiguous", flush=True)
+    _ok(L.lib().ti_linear_i8_residual_f32(ca.data_ptr(), K, cw.data_ptr(), K, cb.data_ptr(), alpha.data_ptr(), beta.data_ptr(), cr.data_ptr(), N,
+                                          hw2.ptr, N, M, N, K, _stream()), "ti_linear_i8_residual_f32")
+    assert hc.surroundings_intact() and hw2.surroundings_intact()
+    assert torch.equal(hc.view, hw2.view) and not torch.isnan(hc.view).any()
+    acc = a.double() @ w.double().t()
+    want = ((acc.float() * 3e-4) + bias.float()) + res  # the three fp32 steps of the contract
+    assert torch.equal(hc.view.cpu(), want)

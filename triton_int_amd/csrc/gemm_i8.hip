@@ -50,7 +50,7 @@ struct GemmParams {
   // bias elements [b * bias_bs, b * bias_bs + N) and the scalars alpha[b * scale_bs], beta[b * scale_bs]
   int64_t bias_bs;
   int64_t scale_bs;
-  // fp32 outputs of gemm_rows4_kernel only: C = epilogue value + resid[m * resid_rs + n]
+  // fp32 outputs of gemm_rows4_kernel and of the persistent kernels' fp32 epilogue: C = epilogue value + resid[m * resid_rs + n]
   const float* resid;
   int64_t resid_rs;
   // int8 outputs of a grouped q/k/v launch of gemm_rows4_kernel only: batch 1 (k) also goes to
@@ -837,6 +837,58 @@ __device__ __forceinline__ void stream_epilogue(const GemmParams& p, const EpiCt
                 const unsigned dword = odd ? (got | (row[1] << 16)) : (row[0] | (got << 16));
                 const int R = i * 32 + 8 * (r >> 2) + (r & 3);  // row mw + R + 4 * lhi + odd
                 __builtin_amdgcn_raw_buffer_store_b32(dword, rC, R < rows_left - odd ? base : OOB, R * pitch, TI_STREAM_STORE32_AUX);
+              }
+            }
+          }
+          return;
+        }
+      }
+      if constexpr (KIND == 2) {
+        if (p.resid) {
+          // fp32 output plus a residual of the same shape (C = epilogue value + resid[m][n], the sum rounded
+          // once more, as the separate addition would): the residual's elements are fetched through a
+          // descriptor of their own with the store's addressing, four rows of the tile at a time and one
+          // group ahead, so that the wait for a group counts only the stores issued since and never waits
+          // for them.
+          const __amdgpu_buffer_rsrc_t rR =
+              __builtin_amdgcn_make_buffer_rsrc((void*)p.resid, 0, ((p.M - 1) * (int)p.resid_rs + p.N) * 4, 0x00020000);
+          const int rpitch = (int)p.resid_rs * 4;
+          float colr[TN];
+          int base_c[TN], base_r[TN];
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+            const int n = nw + j * 32 + lrow;
+            colr[j] = column_term_t<TI_BIAS_F32>(e, min(n, p.N - 1), false);
+            base_c[j] = n < p.N ? ((mw + 4 * lhi) * ldc + n) * ESZ : OOB;
+            base_r[j] = n < p.N ? ((mw + 4 * lhi) * (int)p.resid_rs + n) * 4 : OOB;
+          }
+          constexpr int NG = TM * 4;  // groups of 4 rows: block i, quarter q = r / 4
+          float res[2][4][TN];
+          auto load_group = [&](int g, float (&dst)[4][TN]) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+              const int R = (g >> 2) * 32 + 8 * (g & 3) + t;  // row mw + R + 4 * lhi
+              const bool in = R < rows_left;
+#pragma unroll
+              for (int j = 0; j < TN; ++j)
+                dst[t][j] = __uint_as_float((unsigned)__builtin_amdgcn_raw_buffer_load_b32(rR, in ? base_r[j] : OOB, R * rpitch, 0));
+            }
+          };
+          load_group(0, res[0]);
+#pragma unroll
+          for (int g = 0; g < NG; ++g) {
+            if (g + 1 < NG) load_group(g + 1, res[(g + 1) & 1]);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+              const int R = (g >> 2) * 32 + 8 * (g & 3) + t;
+              const bool in = R < rows_left;
+#pragma unroll
+              for (int j = 0; j < TN; ++j) {
+                float v = (float)acc[g >> 2][j][4 * (g & 3) + t] * e.alpha;
+                const float vb = colr[j] + v;
+                v = has_bias ? vb : v;
+                v = v + res[g & 1][t][j];
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), rC, in ? base_c[j] : OOB, R * pitch, TI_STREAM_STORE32_AUX);
               }
             }
           }
@@ -2720,6 +2772,15 @@ static int run_with_residual(GemmParams p, const float* R, int64_t ldr, hipStrea
     p.resid = R;
     p.resid_rs = ldr;
     return run(p, cfg, stream);
+  }
+  // the persistent kernels add it in their fp32 epilogue (unsplit K only: partial sums carry no residual);
+  // 32-bit offsets into the residual, like the stores
+  const bool persistent = g_configs[cfg].stream_occ > 0 || g_configs[cfg].ws_waves > 0 || g_configs[cfg].max_k > 0;
+  if (persistent && splits == 1 && p.batch == 1 && p.out_dtype == TI_F32 && p.epilogue == TI_EPI_SCALE_F &&
+      ((int64_t)(p.M + 512) * ldr + p.N) * 4 < ((int64_t)1 << 31)) {
+    p.resid = R;
+    p.resid_rs = ldr;
+    return run(p, cfg | (1 << 8), stream);
   }
   rc = run(p, cfg | (splits << 8), stream);
   if (rc != TI_OK) return rc;

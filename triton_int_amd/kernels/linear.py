@@ -70,7 +70,8 @@ def linear_a8_w8_bfp32_ofp32(a, b, bias, scale_a, scale_b, out=None, dtype=None,
 def linear_a8_w8_bfp32_ofp32_residual(a, b, bias, scale_a, scale_b, residual, out=None):
     """`linear_a8_w8_bfp32_ofp32(a, b, bias, scale_a, scale_b) + residual` in fp32 as one library call
     (reference: kernels/linear.py:819-853 followed by the caller's add): with 16 or fewer rows the
-    decode kernel adds the residual while it stores, otherwise an add kernel follows the GEMM.
+    decode kernel adds the residual while it stores, the persistent kernels that serve large outputs add it in
+    their epilogue, otherwise an add kernel follows the GEMM.
     `out` must not overlap `residual`."""
     L.require_cuda(a, b, bias, residual, out)
     assert a.dtype == torch.int8 and b.dtype == torch.int8, "operands must be int8"

@@ -188,7 +188,7 @@ class W8A8OPTDecoderLayer(torch.nn.Module):
         mark("fc1_linear_gelu_q")
         if self.fused_residual and _trace is None:
             y = None
-            out = self.fc2.forward_add(f8, resid)   # decode: one launch; prefill: GEMM + add kernel
+            out = self.fc2.forward_add(f8, resid)   # one launch: the GEMM kernel adds the residual as it stores
             mark("fc2_linear_f32_plus_residual")
         else:
             y = self.fc2(f8)
