@@ -402,7 +402,7 @@ def test_baseline_config2_opt67b_shapes_sampled_rows(which):
 @pytest.mark.parametrize("M,N,K", [(16, 5120, 5120), (1, 5120, 5120), (17, 272, 1040), (48, 100, 64), (64, 20480, 5120), (16, 5120, 20480)])
 def test_decode_shapes_skinny_kernel(M, N, K):
     """M <= 16 takes a weight-streaming kernel (row pieces, or slabs with K split across waves); up to
-    128 rows against a long K take 128 x 128 tiles with K split over workgroups; short K the slabs."""
+    128 rows against a long K take 32 x 128 or 64 x 128 tiles with K split over workgroups; short K the slabs."""
     linear, _, fused = _kl()
     L = _lib()
     g = rng(M * 13 + N)
@@ -412,7 +412,7 @@ def test_decode_shapes_skinny_kernel(M, N, K):
     ga, gw = gpu(a), gpu(w)
     got = cpu(linear.linear_a8_w8_b32_o32(ga, gw, gpu(b32)))
     used = L.lib().ti_gemm_config_name(L.lib().ti_gemm_last_config()).decode()
-    assert used.startswith(("skinny", "rows4") if (M <= 16 or K < 1024) else "ws_128x128"), used
+    assert used.startswith(("skinny", "rows4") if (M <= 16 or K < 1024) else ("ws_32x128" if M <= 32 else "ws_64x128")), used
     assert np.array_equal(got, O.linear_a8_w8_b32_o32(a, w, b32))
     alpha = np.float32(40.0 / (np.sqrt(K) * 127 * 127 / 3)); beta = np.float32(0.05)
     assert np.array_equal(cpu(linear.linear_a8_w8_b8_o8(ga, gw, gpu(b8), alpha, beta)), O.linear_a8_w8_b8_o8(a, w, b8, alpha, beta))

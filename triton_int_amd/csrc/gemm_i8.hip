@@ -2188,6 +2188,8 @@ enum ConfigId {
   CFG_WS_256x160,    // 2048 x 5120 outputs are exactly 256 of these tiles: one full round of the chip
   CFG_WS_128x128,    // few activation rows and a long K: split K over enough of these to fill the chip
   CFG_SHORTK_256x256,  // K <= 128 (attention Q.K^T): a tile's whole K in LDS, one barrier per tile, 128-byte int8 row pieces
+  CFG_WS_64x128,       // 32 < M <= 128 against a long K: six stages of a 64-row tile keep more weight bytes in flight per CU
+  CFG_WS_32x128,       // 16 < M <= 32: seven stages
 };
 
 static const Config g_configs[] = {
@@ -2208,6 +2210,8 @@ static const Config g_configs[] = {
     TI_WS(128, 128, 128, 2, 2, 1, 4, 4),
     {"shortk_256x256x64_w4x2_k128", {gemm_mfma_shortk_kernel<OUT8>, gemm_mfma_shortk_kernel<OUT32>, gemm_mfma_shortk_kernel<OUT16>}, 256, 256, 64, 512,
      true, false, 1, false, 0, 128},
+    TI_WS(64, 128, 128, 2, 2, 1, 6, 4),
+    TI_WS(32, 128, 128, 1, 4, 1, 7, 4),
 };
 static const int g_num_configs = (int)(sizeof(g_configs) / sizeof(g_configs[0]));
 
@@ -2320,12 +2324,16 @@ static int pick_config(const GemmParams& p, int* splits_out) {
   }
   const bool stream = stream_eligible(p);
   if (p.M <= 128 && stream && p.batch == 1 && p.K >= 1024) {
-    // a few rows against a long K: the GEMM is a read of the weight matrix.  128 x 128 tiles with K
-    // split over enough workgroups to have every CU pulling its own slab keep the most weight bytes
-    // in flight (measured, weights from HBM, N = 6848, K = 10240: M = 64 55 -> 29 us against the
-    // 16-row slabs, M = 128 52 -> 28 us against 64 x 64 tiles)
-    *splits_out = pick_splits(p, g_configs[CFG_WS_128x128], 1.0, nullptr);
-    return CFG_WS_128x128;
+    // a few rows against a long K: the GEMM is a read of the weight matrix, and what decides its speed is how
+    // many weight bytes a CU keeps in flight.  K is split over enough workgroups to have every CU pulling its
+    // own slab, and the tile has no more activation rows than needed, so that the LDS holds more stages of
+    // weights: 32 x 128 tiles with 7 stages up to 32 rows, 64 x 128 with 6 stages beyond (a 128 x 128 tile has
+    // room for 4).  Measured in steady state, weights rotated through 350 MB, N = 6848, K = 10240, against
+    // the 128 x 128 tile: M = 17 .. 32 34 -> 22-23 us, M = 64 35 -> 28.5 us, M = 128 38 -> 33 us; N = K = 5120:
+    // 18.5-19 -> 15-16 us, M = 128 20.4 -> 16.6 us.
+    const int cfg = p.M <= 32 ? CFG_WS_32x128 : CFG_WS_64x128;
+    *splits_out = pick_splits(p, g_configs[cfg], 1.0, nullptr);
+    return cfg;
   }
   if (p.M <= 64) return CFG_SKINNY_16 + (p.M > 16) + (p.M > 32);
   // K <= 128, int8 out, at least two 256 x 256 tiles per workgroup: the epilogue is most of the work
